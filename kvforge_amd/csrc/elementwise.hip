@@ -1,0 +1,207 @@
+// Row-wise kernels of the decoder: embedding gather, RMS norm, SwiGLU gate, rotary + cache write.
+// The residual stream is fp32 in every mode; T is the activation / weight element type.
+#include "common.h"
+
+// ----------------------------------------------------------------------------- embedding
+// out[n, :] = table[ids[n], :] widened to fp32.  An id outside [0, vocab) writes zeros.
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ out, int h, int vocab) {
+  const int n = blockIdx.x;
+  const int id = ids[n];
+  float* o = out + static_cast<size_t>(n) * h;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = 0.f;
+    return;
+  }
+  const T* row = table + static_cast<size_t>(id) * h;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = Elem<T>::load(row + i);
+}
+
+template <typename T>
+static int embed_launch(const int* ids, const void* table, float* out, int n, int h, int vocab,
+                        hipStream_t s) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(embed_kernel<T>, dim3(n), dim3(256), 0, s, ids, static_cast<const T*>(table),
+                     out, h, vocab);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_embed_f32(const int* ids, const void* t, float* o, int n, int h, int v,
+                             hipStream_t s) { return embed_launch<float>(ids, t, o, n, h, v, s); }
+KVF_EXPORT int kvf_embed_bf16(const int* ids, const void* t, float* o, int n, int h, int v,
+                              hipStream_t s) { return embed_launch<bf16_t>(ids, t, o, n, h, v, s); }
+
+// ----------------------------------------------------------------------------- RMS norm
+// y = x * rsqrt(mean(x^2) + eps) * w, all in fp32, rounded once to T on store.
+// x is the fp32 residual stream; `rows` (may be null) gathers input rows; w is fp32 or T.
+template <typename T, typename W>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                               const W* __restrict__ w, float eps, T* __restrict__ out, int h,
+                               int x_rows) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  int src = rows ? rows[m] : m;
+  T* o = out + static_cast<size_t>(m) * h;
+  if (src < 0 || src >= x_rows) {
+    for (int i = threadIdx.x; i < h; i += blockDim.x) Elem<T>::store(o + i, 0.f);
+    return;
+  }
+  const float* xr = x + static_cast<size_t>(src) * h;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    const float v = xr[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = rsqrtf(ss / static_cast<float>(h) + eps);
+  for (int i = threadIdx.x; i < h; i += blockDim.x)
+    Elem<T>::store(o + i, xr[i] * r * Elem<W>::load(w + i));
+}
+
+template <typename T>
+static int rmsnorm_launch(const float* x, const int* rows, const void* w, int w_is_f32, float eps,
+                          void* out, int m, int h, int x_rows, hipStream_t s) {
+  if (m <= 0) return 0;
+  const int threads = h >= 1024 ? 256 : (h >= 256 ? 128 : 64);
+  if (w_is_f32)
+    hipLaunchKernelGGL((rmsnorm_kernel<T, float>), dim3(m), dim3(threads), 0, s, x, rows,
+                       static_cast<const float*>(w), eps, static_cast<T*>(out), h, x_rows);
+  else
+    hipLaunchKernelGGL((rmsnorm_kernel<T, T>), dim3(m), dim3(threads), 0, s, x, rows,
+                       static_cast<const T*>(w), eps, static_cast<T*>(out), h, x_rows);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_rmsnorm_f32(const float* x, const int* rows, const void* w, int wf, float eps,
+                               void* out, int m, int h, int xr, hipStream_t s) {
+  return rmsnorm_launch<float>(x, rows, w, wf, eps, out, m, h, xr, s);
+}
+KVF_EXPORT int kvf_rmsnorm_bf16(const float* x, const int* rows, const void* w, int wf, float eps,
+                                void* out, int m, int h, int xr, hipStream_t s) {
+  return rmsnorm_launch<bf16_t>(x, rows, w, wf, eps, out, m, h, xr, s);
+}
+
+// ----------------------------------------------------------------------------- SwiGLU gate
+// out[m, i] = silu(gu[m, i]) * gu[m, I + i], silu(x) = x / (1 + exp(-x)), in fp32.
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter,
+                                size_t total) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / inter;
+  const int i = static_cast<int>(idx - m * inter);
+  const T* row = gu + m * 2 * static_cast<size_t>(inter);
+  const float g = Elem<T>::load(row + i);
+  const float u = Elem<T>::load(row + inter + i);
+  Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
+}
+template <typename T>
+static int silu_mul_launch(const void* gu, void* out, int m, int inter, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * inter;
+  if (total == 0) return 0;
+  const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+  hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, s,
+                     static_cast<const T*>(gu), static_cast<T*>(out), inter, total);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_silu_mul_f32(const void* gu, void* out, int m, int inter, hipStream_t s) {
+  return silu_mul_launch<float>(gu, out, m, inter, s);
+}
+KVF_EXPORT int kvf_silu_mul_bf16(const void* gu, void* out, int m, int inter, hipStream_t s) {
+  return silu_mul_launch<bf16_t>(gu, out, m, inter, s);
+}
+
+// ----------------------------------------------------------------------------- rotary + cache write
+// qkv: [N, (H + 2*KV) * d] rows of q heads, then k heads, then v heads.
+// For token n at position p (cos/sin tables [table_len, rot/2] fp32):
+//   q and k: x'[i] = x[i]*cos[i] - x[i+rot/2]*sin[i];  x'[i+rot/2] = x[i+rot/2]*cos[i] + x[i]*sin[i]
+//   for i < rot/2; elements at or beyond `rot` are copied.  q is rotated in place.
+// Rotated k and v go to the pages: page = block_table[seq_of_token[n], p / block_size];
+// a negative page (padding, or a page already given back) or p outside the table skips the write.
+// Pages are [num_blocks, KV, block_size, d].  With write_kv == 0 only q is rotated.
+struct RopeArgs {
+  int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
+};
+
+template <typename T>
+__global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                    const int* __restrict__ seq_of_token,
+                                    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                    const int* __restrict__ block_table, T* __restrict__ k_pages,
+                                    T* __restrict__ v_pages, RopeArgs a) {
+  const int n = blockIdx.x;
+  const int p = positions[n];
+  const int half = a.rot / 2;
+  T* row = qkv + static_cast<size_t>(n) * (a.H + 2 * a.KV) * a.d;
+  const bool pos_ok = p >= 0 && p < a.table_len;
+  const float* cs = cos_t + static_cast<size_t>(pos_ok ? p : 0) * half;
+  const float* sn = sin_t + static_cast<size_t>(pos_ok ? p : 0) * half;
+
+  int page = -1, off = 0;
+  if (a.write_kv && pos_ok) {
+    const int seq = seq_of_token[n];
+    const int blk = p / a.block_size;
+    if (seq >= 0 && seq < a.n_seqs && blk < a.table_stride) {
+      page = block_table[static_cast<size_t>(seq) * a.table_stride + blk];
+      if (page >= a.num_blocks) page = -1;
+      off = p - blk * a.block_size;
+    }
+  }
+  // q heads: rotate in place (pairs are owned by one thread, so no hazard)
+  const int q_pairs = a.H * half;
+  for (int t = threadIdx.x; t < q_pairs; t += blockDim.x) {
+    const int hh = t / half, i = t - hh * half;
+    T* x = row + hh * a.d;
+    const float x1 = Elem<T>::load(x + i), x2 = Elem<T>::load(x + i + half);
+    const float c = pos_ok ? cs[i] : 1.f, s = pos_ok ? sn[i] : 0.f;
+    Elem<T>::store(x + i, x1 * c - x2 * s);
+    Elem<T>::store(x + i + half, x2 * c + x1 * s);
+  }
+  if (page < 0) return;
+  // k heads: rotate, write to the page; the unrotated tail is copied
+  const int k_pairs = a.KV * half;
+  for (int t = threadIdx.x; t < k_pairs; t += blockDim.x) {
+    const int hh = t / half, i = t - hh * half;
+    const T* x = row + (a.H + hh) * a.d;
+    T* dst = k_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d;
+    const float x1 = Elem<T>::load(x + i), x2 = Elem<T>::load(x + i + half);
+    Elem<T>::store(dst + i, x1 * cs[i] - x2 * sn[i]);
+    Elem<T>::store(dst + i + half, x2 * cs[i] + x1 * sn[i]);
+  }
+  const int tail = a.d - a.rot;
+  for (int t = threadIdx.x; t < a.KV * tail; t += blockDim.x) {
+    const int hh = t / tail, i = a.rot + (t - hh * tail);
+    T* dst = k_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d;
+    dst[i] = row[(a.H + hh) * a.d + i];
+  }
+  for (int t = threadIdx.x; t < a.KV * a.d; t += blockDim.x) {
+    const int hh = t / a.d, i = t - hh * a.d;
+    T* dst = v_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d;
+    dst[i] = row[(a.H + a.KV + hh) * a.d + i];
+  }
+}
+
+template <typename T>
+static int rope_launch(void* qkv, const int* positions, const int* seq_of_token, const float* cos_t,
+                       const float* sin_t, const int* block_table, void* k_pages, void* v_pages,
+                       int n, RopeArgs a, hipStream_t s) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(rope_kvwrite_kernel<T>, dim3(n), dim3(128), 0, s, static_cast<T*>(qkv),
+                     positions, seq_of_token, cos_t, sin_t, block_table, static_cast<T*>(k_pages),
+                     static_cast<T*>(v_pages), a);
+  return kvf_last_error();
+}
+#define ROPE_ARGS_DECL                                                                           \
+  void *qkv, const int *positions, const int *seq_of_token, const float *cos_t,                 \
+      const float *sin_t, const int *block_table, void *k_pages, void *v_pages, int n, int H,   \
+      int KV, int d, int rot, int table_len, int block_size, int table_stride, int num_blocks,  \
+      int write_kv, int n_seqs, hipStream_t s
+#define ROPE_ARGS_PACK                                                                           \
+  RopeArgs { H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs }
+KVF_EXPORT int kvf_rope_kvwrite_f32(ROPE_ARGS_DECL) {
+  return rope_launch<float>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
+                            v_pages, n, ROPE_ARGS_PACK, s);
+}
+KVF_EXPORT int kvf_rope_kvwrite_bf16(ROPE_ARGS_DECL) {
+  return rope_launch<bf16_t>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
+                             v_pages, n, ROPE_ARGS_PACK, s);
+}

@@ -1,0 +1,111 @@
+// C[M, N] = A[M, K] * W[N, K]^T with fp32 multiply and fp32 accumulate on the vector ALUs.
+// This is the matrix product of the true 32-bit path and the fallback for operand types the
+// MFMA kernels do not take (for instance a weight that the checkpoint stores in fp32 while
+// activations are bf16).  No reduced-precision matrix instruction is used.
+//
+// Each output element is accumulated over k = 0..K-1 in one fixed order by one thread, so a
+// row's result does not depend on M, on the row's place in the batch or on the grid.
+//
+// Output modes: 0 = store as TO;  1 = add into a fp32 matrix (the residual stream).
+#include "common.h"
+
+namespace {
+constexpr int BM = 64, BN = 64, BK = 16, TM = 4, TN = 4;
+
+template <typename TA, typename TW, typename TO, int MODE>
+__global__ __launch_bounds__(256) void gemm_tile_kernel(const TA* __restrict__ A,
+                                                        const TW* __restrict__ W,
+                                                        TO* __restrict__ C, int M, int N, int K,
+                                                        int lda, int ldc) {
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int tr = tid / 16, tc = tid % 16;  // micro-tile rows tr*4.., cols tc*4..
+  float acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
+
+  const int lrow = tid / 4, lk = (tid % 4) * 4;  // this thread stages 4 consecutive k of one row
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    {
+      const int m = m0 + lrow;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int k = k0 + lk + e;
+        As[lk + e][lrow] = (m < M && k < K) ? Elem<TA>::load(A + static_cast<size_t>(m) * lda + k)
+                                            : 0.f;
+      }
+      const int n = n0 + lrow;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int k = k0 + lk + e;
+        Ws[lk + e][lrow] = (n < N && k < K) ? Elem<TW>::load(W + static_cast<size_t>(n) * K + k)
+                                            : 0.f;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[TM], w[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = As[kk][tr * TM + i];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) w[j] = Ws[kk][tc * TN + j];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + tr * TM + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + tc * TN + j;
+      if (n >= N) continue;
+      TO* c = C + static_cast<size_t>(m) * ldc + n;
+      if (MODE == 1) {
+        Elem<TO>::store(c, Elem<TO>::load(c) + acc[i][j]);
+      } else {
+        Elem<TO>::store(c, acc[i][j]);
+      }
+    }
+  }
+}
+
+template <typename TA, typename TW, typename TO, int MODE>
+int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
+           hipStream_t s) {
+  if (M <= 0 || N <= 0) return 0;
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+  hipLaunchKernelGGL((gemm_tile_kernel<TA, TW, TO, MODE>), grid, dim3(256), 0, s,
+                     static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C), M,
+                     N, K, lda, ldc);
+  return kvf_last_error();
+}
+}  // namespace
+
+// a_type / w_type: 0 = fp32, 1 = bf16.  out_mode: 0 = store in a_type... see table below.
+//   out_kind 0: store fp32      out_kind 1: store bf16      out_kind 2: add into fp32
+KVF_EXPORT int kvf_gemm_generic(const void* A, int a_type, const void* W, int w_type, void* C,
+                                int out_kind, int M, int N, int K, int lda, int ldc,
+                                hipStream_t s) {
+#define CASE(AT, WT, TA, TW)                                                                      \
+  if (a_type == AT && w_type == WT) {                                                             \
+    if (out_kind == 0) return launch<TA, TW, float, 0>(A, W, C, M, N, K, lda, ldc, s);            \
+    if (out_kind == 1) return launch<TA, TW, bf16_t, 0>(A, W, C, M, N, K, lda, ldc, s);           \
+    if (out_kind == 2) return launch<TA, TW, float, 1>(A, W, C, M, N, K, lda, ldc, s);            \
+  }
+  CASE(0, 0, float, float)
+  CASE(0, 1, float, bf16_t)
+  CASE(1, 0, bf16_t, float)
+  CASE(1, 1, bf16_t, bf16_t)
+#undef CASE
+  return static_cast<int>(hipErrorInvalidValue);
+}

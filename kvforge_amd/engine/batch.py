@@ -1,0 +1,255 @@
+"""The flat batch of one step: entries (request, its next tokens, where they start, which logits
+are wanted) become int32 arrays in one fixed-address device buffer.
+
+This is the reference's ``BatchItem`` / ``prepare_inputs`` (src/tokenvault/batching/continuous.py:
+27-87) with two differences: there is no per-token slot list (kernels compute a token's slot from
+its sequence's block-table row and its position), and sequences are told apart into query runs
+(more than one token, prefill kernel) and single tokens (decode kernel) while the matrix products
+still see one ``[N, hidden]`` matrix.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Sequence
+
+import numpy as np
+import torch
+
+ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup handles
+
+
+@dataclass
+class StepEntry:
+    """``want``: places among ``token_ids`` whose logits are returned, or ``"last"`` / ``"all"``
+    / ``"none"`` (the reference's ``LogitsMode``)."""
+
+    request_id: str
+    token_ids: Sequence[int]
+    start_pos: int
+    want: "Sequence[int] | str" = "last"
+
+    def wanted(self) -> list[int]:
+        n = len(self.token_ids)
+        if isinstance(self.want, str):
+            if self.want == "last":
+                return [n - 1]
+            if self.want == "all":
+                return list(range(n))
+            if self.want == "none":
+                return []
+            raise ValueError(f"unknown logits mode {self.want!r}")
+        out = [int(i) for i in self.want]
+        for i in out:
+            if not 0 <= i < n:
+                raise ValueError(f"wanted place {i} outside the entry's {n} tokens")
+        return out
+
+
+class Workspace:
+    """Named scratch tensors that live across steps and grow on demand."""
+
+    def __init__(self, device: torch.device | str) -> None:
+        self.device = device
+        self._bufs: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+        self.frozen = False
+
+    def buf(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        flat = self._bufs.get(key)
+        if flat is None or flat.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"workspace buffer {name} would grow during graph capture")
+            flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = flat
+        return flat[:n].view(shape)
+
+    def snapshot(self) -> list[torch.Tensor]:
+        return list(self._bufs.values())
+
+
+class MetaBuffers:
+    """Fixed-address int32 device memory for batch metadata, filled through pinned staging."""
+
+    def __init__(self, max_tokens: int, max_seqs: int, table_widths: list[int],
+                 device: torch.device | str) -> None:
+        self.max_tokens, self.max_seqs, self.table_widths = max_tokens, max_seqs, list(table_widths)
+        off = 0
+        self.off: dict[str, int] = {}
+        for name, size in (("cu_q", max_seqs + 1), ("ctx_lens", max_seqs), ("slot_ids", max_seqs),
+                           ("decode_seq_ids", max_seqs), ("token_ids", max_tokens),
+                           ("positions", max_tokens), ("seq_of_token", max_tokens),
+                           ("logits_rows", max_tokens)):
+            self.off[name] = off
+            off += (size + 3) // 4 * 4
+        self.table_off: list[int] = []
+        for w in self.table_widths:
+            self.table_off.append(off)
+            off += max_seqs * w
+        self.total = off
+        self.device_buf = torch.zeros(self.total, dtype=torch.int32, device=device)
+        pin = torch.device(device).type == "cuda"
+        self.staging = [torch.zeros(self.total, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self.staging_np = [s.numpy() for s in self.staging]
+        self.events: list[torch.cuda.Event | None] = [None, None]
+        self.turn = 0
+
+    def view(self, name: str, n: int) -> torch.Tensor:
+        o = self.off[name]
+        return self.device_buf[o:o + n]
+
+    def table_view(self, g: int) -> torch.Tensor:
+        o, w = self.table_off[g], self.table_widths[g]
+        return self.device_buf[o:o + self.max_seqs * w].view(self.max_seqs, w)
+
+
+class Step:
+    """One step's batch on the device, plus the host-side facts parts may need."""
+
+    def __init__(self) -> None:
+        self.n_tokens = 0
+        self.n_seqs = 0
+        self.n_logits = 0
+        self.n_decode = 0
+        self.act_dtype: torch.dtype = torch.float32
+        self.ws: Workspace = None  # type: ignore[assignment]
+        self.token_ids = self.positions = self.seq_of_token = None
+        self.cu_q = self.ctx_lens = self.slot_ids = self.logits_rows = None
+        self.decode_seq_ids: torch.Tensor | None = None
+        self.block_tables: list[torch.Tensor] = []
+        # host copies
+        self.request_ids: list[str] = []
+        self.q_lens: list[int] = []
+        self.start_pos: list[int] = []
+        self.host_slot_ids: list[int] = []
+        self.host_token_ids: np.ndarray | None = None
+        self.prefill_seqs: list[int] = []
+        self.max_decode_ctx = 0
+        self._work: dict[int, torch.Tensor | None] = {}
+        self._identity_rotary = None
+        self.device: torch.device | str = "cuda"
+
+    def prefill_work(self, group_size: int) -> torch.Tensor | None:
+        """``[num_work, 2]`` (sequence row, 16-row tile) for every query run longer than one
+        token, given ``group_size`` query heads per kv head."""
+        if not self.prefill_seqs:
+            return None
+        w = self._work.get(group_size)
+        if w is None:
+            pairs = [(b, t) for b in self.prefill_seqs
+                     for t in range(-(-self.q_lens[b] * group_size // ROWS_PER_TILE))]
+            w = torch.tensor(pairs, dtype=torch.int32).reshape(-1, 2).to(self.device)
+            self._work[group_size] = w
+        return w
+
+    def decode_plan(self, H: int, KV: int, d: int, window: int):
+        """How many splits of the key range the decode kernel uses, and its workspace."""
+        G = H // KV
+        chunks = -(-G // (4 if G <= 4 else 8))
+        wgs = max(1, self.n_decode * KV * chunks)
+        ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
+        splits = 1
+        if wgs < 256:
+            splits = max(1, min(-(-512 // wgs), ctx // 256, 64))
+        if splits == 1:
+            return 1, None
+        acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)
+        ml = self.ws.buf("decode_part_ml", (self.n_decode * H * splits * 2,), torch.float32)
+        return splits, (acc, ml)
+
+
+def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], tables_of, slot_of,
+              block_size: int, pad_to: int | None = None) -> list[int]:
+    """Write the batch into ``meta`` (one host-to-device copy) and point ``step`` at it.
+    ``tables_of(request_id, group) -> list[int]``; ``slot_of(request_id) -> int``.
+    ``pad_to``: pad a pure-decode batch with empty sequences up to this many.
+    Returns how many logits rows each entry gets."""
+    B = len(entries)
+    q_lens = [len(e.token_ids) for e in entries]
+    if B == 0 or min(q_lens) <= 0:
+        raise ValueError("a step needs entries, each with at least one token")
+    Bp = B if pad_to is None else int(pad_to)
+    N = sum(q_lens) + (Bp - B)
+    if Bp > meta.max_seqs or N > meta.max_tokens:
+        raise ValueError(f"step of {N} tokens / {Bp} requests exceeds the runner's capacity "
+                         f"({meta.max_tokens} tokens / {meta.max_seqs} requests)")
+    turn = meta.turn
+    meta.turn ^= 1
+    if meta.events[turn] is not None:
+        meta.events[turn].synchronize()
+    host = meta.staging_np[turn]
+    off = meta.off
+
+    lens = np.asarray(q_lens + [1] * (Bp - B), dtype=np.int32)
+    starts = np.asarray([e.start_pos for e in entries] + [0] * (Bp - B), dtype=np.int32)
+    cu = np.zeros(Bp + 1, dtype=np.int32)
+    np.cumsum(lens, out=cu[1:])
+    host[off["cu_q"]:off["cu_q"] + Bp + 1] = cu
+    ctx = starts + lens
+    ctx[B:] = 0  # padding sequences hold nothing
+    host[off["ctx_lens"]:off["ctx_lens"] + Bp] = ctx
+    slots = [slot_of(e.request_id) for e in entries] + [-1] * (Bp - B)
+    host[off["slot_ids"]:off["slot_ids"] + Bp] = slots
+    tok = host[off["token_ids"]:off["token_ids"] + N]
+    pos = host[off["positions"]:off["positions"] + N]
+    p = 0
+    for e, n, s in zip(entries, q_lens, starts[:B]):
+        tok[p:p + n] = e.token_ids
+        pos[p:p + n] = np.arange(s, s + n, dtype=np.int32)
+        p += n
+    tok[p:] = 0
+    pos[p:] = 0
+    host[off["seq_of_token"]:off["seq_of_token"] + N] = np.repeat(np.arange(Bp, dtype=np.int32), lens)
+
+    counts, rows = [], []
+    for b, e in enumerate(entries):
+        w = e.wanted()
+        counts.append(len(w))
+        rows.extend(int(cu[b]) + i for i in w)
+    R = len(rows)
+    host[off["logits_rows"]:off["logits_rows"] + R] = rows
+
+    decode = [b for b in range(Bp) if lens[b] == 1]
+    prefill = [b for b in range(B) if lens[b] > 1]
+    host[off["decode_seq_ids"]:off["decode_seq_ids"] + len(decode)] = decode
+
+    end = off["logits_rows"] + max(R, 1)
+    for g, (to, w) in enumerate(zip(meta.table_off, meta.table_widths)):
+        tab = host[to:to + Bp * w].reshape(Bp, w)
+        tab[:] = -1
+        for b, e in enumerate(entries):
+            t = tables_of(e.request_id, g)
+            need = -(-int(ctx[b]) // block_size)
+            if need > w or need > len(t):
+                raise ValueError(f"request {e.request_id} needs {need} pages in group {g}; "
+                                 f"table holds {len(t)}, width {w}")
+            tab[b, :need] = t[:need]
+        end = to + Bp * w
+    meta.device_buf[:end].copy_(meta.staging[turn][:end], non_blocking=True)
+    if meta.device_buf.is_cuda:
+        ev = meta.events[turn] or torch.cuda.Event()
+        ev.record()
+        meta.events[turn] = ev
+
+    step.n_tokens, step.n_seqs, step.n_logits, step.n_decode = N, Bp, R, len(decode)
+    step.token_ids = meta.view("token_ids", N)
+    step.positions = meta.view("positions", N)
+    step.seq_of_token = meta.view("seq_of_token", N)
+    step.cu_q = meta.view("cu_q", Bp + 1)
+    step.ctx_lens = meta.view("ctx_lens", Bp)
+    step.slot_ids = meta.view("slot_ids", Bp)
+    step.logits_rows = meta.view("logits_rows", max(R, 1))[:R]
+    step.decode_seq_ids = None if len(decode) == Bp else meta.view("decode_seq_ids", len(decode))
+    step.block_tables = [meta.table_view(g)[:Bp] for g in range(len(meta.table_widths))]
+    step.request_ids = [e.request_id for e in entries]
+    step.q_lens = [int(x) for x in lens]
+    step.start_pos = [int(x) for x in starts]
+    step.host_slot_ids = slots
+    step.host_token_ids = tok.copy()
+    step.prefill_seqs = prefill
+    step.max_decode_ctx = int(max((ctx[b] for b in decode), default=0))
+    step._work = {}
+    return counts

@@ -1,0 +1,303 @@
+"""Python faces of the HIP kernels.  Each function checks on the host that shapes, dtypes,
+devices and strides are what its kernel and launch grid assume, then launches on torch's
+current stream (so launches made while a torch HIP-graph capture is active are captured).
+
+There is no fallback: every function here runs a hand-written gfx950 kernel or raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_void_p
+
+import torch
+
+from kvforge_amd.kernels import library
+
+F32, BF16, I32 = torch.float32, torch.bfloat16, torch.int32
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _tcode(dtype: torch.dtype) -> int:
+    if dtype == F32:
+        return 0
+    if dtype == BF16:
+        return 1
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {dtype}")
+
+
+def _suffix(dtype: torch.dtype) -> str:
+    return "f32" if _tcode(dtype) == 0 else "bf16"
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name} must be a tensor on the GPU")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and int(s) != int(ts)
+                                        for s, ts in zip(shape, t.shape)):
+            raise KernelError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+    if contiguous and not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+
+
+def _ok(code: int, what: str) -> None:
+    if code != 0:
+        raise KernelError(f"{what} failed with HIP error {code}")
+
+
+_fn_cache: dict[tuple[str, str], object] = {}
+
+
+def _fn(module: str, name: str, argtypes: list):
+    key = (module, name)
+    f = _fn_cache.get(key)
+    if f is None:
+        lib = library.load(module)
+        try:
+            f = getattr(lib, name)
+        except AttributeError:
+            raise KernelError(f"kernel module {module!r} has no entry point {name!r}") from None
+        f.argtypes = argtypes
+        f.restype = c_int
+        _fn_cache[key] = f
+    return f
+
+
+# ------------------------------------------------------------------------------ embedding
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[n] = table[ids[n]]`` widened to fp32 (the residual stream)."""
+    n = ids.shape[0]
+    _check(ids, "ids", I32, (n,))
+    _check(table, "table", None, (None, None))
+    vocab, h = table.shape
+    _check(out, "out", F32, (n, h))
+    f = _fn("elementwise", f"kvf_embed_{_suffix(table.dtype)}",
+            [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p])
+    _ok(f(ids.data_ptr(), table.data_ptr(), out.data_ptr(), n, h, vocab, _stream()), "embed")
+
+
+# ------------------------------------------------------------------------------ RMS norm
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: torch.Tensor | None = None) -> None:
+    """``out[m] = x[rows[m] or m] * rsqrt(mean(x^2) + eps) * weight`` with fp32 math."""
+    _check(x, "x", F32, (None, None))
+    xr, h = x.shape
+    m = out.shape[0]
+    _check(out, "out", None, (m, h))
+    _check(weight, "weight", None, (h,))
+    if weight.dtype not in (F32, out.dtype):
+        raise KernelError(f"norm weight must be float32 or {out.dtype}, got {weight.dtype}")
+    if rows is not None:
+        _check(rows, "rows", I32, (m,))
+    elif m > xr:
+        raise KernelError("rmsnorm: more output rows than input rows")
+    f = _fn("elementwise", f"kvf_rmsnorm_{_suffix(out.dtype)}",
+            [c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), rows.data_ptr() if rows is not None else None, weight.data_ptr(),
+          1 if weight.dtype == F32 else 0, float(eps), out.data_ptr(), m, h, xr, _stream()),
+        "rmsnorm")
+
+
+# ------------------------------------------------------------------------------ SwiGLU gate
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = silu(gate_up[:, :I]) * gate_up[:, I:]``."""
+    m, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("silu_mul: input width must be even")
+    _check(gate_up, "gate_up", None, (m, two_i))
+    _check(out, "out", gate_up.dtype, (m, two_i // 2))
+    f = _fn("elementwise", f"kvf_silu_mul_{_suffix(out.dtype)}",
+            [c_void_p, c_void_p, c_int, c_int, c_void_p])
+    _ok(f(gate_up.data_ptr(), out.data_ptr(), m, two_i // 2, _stream()), "silu_mul")
+
+
+# ------------------------------------------------------------------------------ rotary + cache
+def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                 cos: torch.Tensor, sin: torch.Tensor, block_table: torch.Tensor,
+                 k_pages: torch.Tensor, v_pages: torch.Tensor, num_heads: int, num_kv_heads: int,
+                 head_dim: int, write_kv: bool = True) -> None:
+    """Rotate q (in place) and k by the cos/sin rows of each token's position; write rotated k
+    and v into the pages named by the token's sequence row of ``block_table``."""
+    n = qkv.shape[0]
+    H, KV, d = num_heads, num_kv_heads, head_dim
+    _check(qkv, "qkv", None, (n, (H + 2 * KV) * d))
+    _check(positions, "positions", I32, (None,))
+    _check(seq_of_token, "seq_of_token", I32, (None,))
+    if positions.shape[0] < n or seq_of_token.shape[0] < n:
+        raise KernelError("rope_kvwrite: positions / seq_of_token shorter than the batch")
+    _check(cos, "cos", F32, (None, None))
+    _check(sin, "sin", F32, tuple(cos.shape))
+    table_len, half = cos.shape
+    rot = 2 * half
+    if rot > d or rot <= 0:
+        raise KernelError(f"rope_kvwrite: rotary width {rot} does not fit head_dim {d}")
+    _check(block_table, "block_table", I32, (None, None))
+    n_seqs, stride = block_table.shape
+    _check(k_pages, "k_pages", qkv.dtype, (None, KV, None, d))
+    _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
+    nb, _, bs, _ = k_pages.shape
+    f = _fn("elementwise", f"kvf_rope_kvwrite_{_suffix(qkv.dtype)}",
+            [c_void_p] * 8 + [c_int] * 11 + [c_void_p])
+    _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(),
+          sin.data_ptr(), block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+          n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs, _stream()),
+        "rope_kvwrite")
+
+
+# ------------------------------------------------------------------------------ matrix products
+_OUT_KIND = {"f32": 0, "bf16": 1, "add": 2}
+
+# Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.
+SKINNY_MAX_M = 128
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``out = a @ w.T`` (``accumulate``: ``out += a @ w.T`` with ``out`` fp32).
+
+    ``a: [M, K]`` (row stride may exceed K), ``w: [N, K]`` contiguous, ``out: [M, N]``.
+    bf16 x bf16 runs on MFMA with fp32 accumulation; any operand in fp32 runs the fp32
+    vector-ALU kernel (true 32-bit multiply and accumulate)."""
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+        raise KernelError("gemm takes 2-D tensors")
+    m, k = a.shape
+    n, k2 = w.shape
+    if k != k2 or tuple(out.shape) != (m, n):
+        raise KernelError(f"gemm shapes do not agree: a {list(a.shape)}, w {list(w.shape)}, "
+                          f"out {list(out.shape)}")
+    _check(a, "a", None, None, contiguous=False)
+    _check(w, "w")
+    _check(out, "out", None, None, contiguous=False)
+    if a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: rows of a and out must be dense")
+    if accumulate and out.dtype != F32:
+        raise KernelError("gemm: accumulation needs an fp32 output")
+    if m == 0:
+        return
+    lda, ldc = a.stride(0) if m > 1 else k, out.stride(0) if m > 1 else n
+    out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)
+    if not accumulate:
+        _tcode(out.dtype)
+    if a.dtype == BF16 and w.dtype == BF16 and _bf16_gemm_ok(m, n, k, lda, ldc):
+        f = _fn("gemm_bf16", "kvf_gemm_bf16", [c_void_p, c_void_p, c_void_p] + [c_int] * 6 + [c_void_p])
+        _ok(f(a.data_ptr(), w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc, _stream()),
+            "gemm_bf16")
+        return
+    f = _fn("gemm_generic", "kvf_gemm_generic",
+            [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_void_p])
+    _ok(f(a.data_ptr(), _tcode(a.dtype), w.data_ptr(), _tcode(w.dtype), out.data_ptr(), out_kind,
+          m, n, k, lda, ldc, _stream()), "gemm_generic")
+
+
+def _bf16_gemm_ok(m: int, n: int, k: int, lda: int, ldc: int) -> bool:
+    """The MFMA kernels need K in steps of 32 and 16-byte aligned rows."""
+    return ("gemm_bf16" in library.available_modules() and k % 32 == 0 and lda % 8 == 0
+            and n % 16 == 0)
+
+
+# ------------------------------------------------------------------------------ attention
+def _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d):
+    if d % 16 or d > 256 or d <= 0:
+        raise KernelError(f"attention kernels take head sizes in steps of 16 up to 256, got {d}")
+    if H % KV:
+        raise KernelError(f"query heads ({H}) must be a multiple of kv heads ({KV})")
+    _check(q, "q", None, (None, None), contiguous=False)
+    if q.stride(1) != 1 or q.shape[1] < H * d:
+        raise KernelError("attention: q rows must be dense and hold all query heads")
+    _check(k_pages, "k_pages", q.dtype, (None, KV, None, d))
+    _check(v_pages, "v_pages", q.dtype, tuple(k_pages.shape))
+    _check(block_table, "block_table", I32, (None, None))
+    n_seqs = block_table.shape[0]
+    _check(cu_q, "cu_q", I32, (None,))
+    _check(ctx_lens, "ctx_lens", I32, (None,))
+    if cu_q.shape[0] < n_seqs + 1 or ctx_lens.shape[0] < n_seqs:
+        raise KernelError("attention: cu_q / ctx_lens shorter than the block table")
+    _check(out, "out", q.dtype, (None, H * d))
+    if out.shape[0] < q.shape[0]:
+        raise KernelError("attention: out has fewer rows than q")
+    return n_seqs
+
+
+def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                 block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
+                 work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
+                 head_dim: int, scale: float, window: int = 0, force_generic: bool = False) -> None:
+    """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 2]`` pairs
+    (sequence row, tile of 16 rows) where a sequence has ``query_len * H/KV`` rows per kv head."""
+    H, KV, d = num_heads, num_kv_heads, head_dim
+    n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    _check(work, "work", I32, (None, 2))
+    nb, _, bs, _ = k_pages.shape
+    f = _fn("attn_generic", "kvf_attn_generic",
+            [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p])
+    _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+          block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
+          work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
+          out.stride(0), int(window), n_seqs, float(scale), _stream()), "attn_generic")
+
+
+def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                block_table: torch.Tensor, seq_ids: torch.Tensor | None, num_seqs: int,
+                cu_q: torch.Tensor, ctx_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
+                num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
+                workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:
+    """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
+    each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys."""
+    H, KV, d = num_heads, num_kv_heads, head_dim
+    n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    if seq_ids is not None:
+        _check(seq_ids, "seq_ids", I32, (None,))
+        if seq_ids.shape[0] < num_seqs:
+            raise KernelError("attn_decode: seq_ids shorter than num_seqs")
+    elif num_seqs > n_seqs:
+        raise KernelError("attn_decode: more sequences than block-table rows")
+    pa = pm = None
+    if splits > 1:
+        if workspace is None:
+            raise KernelError("attn_decode: splits > 1 need a workspace")
+        pa, pm = workspace
+        _check(pa, "workspace[0]", F32)
+        _check(pm, "workspace[1]", F32)
+        if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
+            raise KernelError("attn_decode: workspace too small")
+    nb, _, bs, _ = k_pages.shape
+    f = _fn("attn_decode", "kvf_attn_decode",
+            [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+    _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+          block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
+          cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
+          pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
+          num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
+          int(window), n_seqs, int(splits), float(scale), _stream()), "attn_decode")
+
+
+# ------------------------------------------------------------------------------ sampling
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None,
+           top_p: torch.Tensor | None, u: torch.Tensor, tokens: torch.Tensor) -> None:
+    """One token per row of fp32 ``logits``: argmax where ``temperature == 0``, otherwise the
+    inverse CDF of the processed distribution at ``u``."""
+    _check(logits, "logits", F32, (None, None), contiguous=False)
+    if logits.stride(1) != 1:
+        raise KernelError("sample: logits rows must be dense")
+    r, v = logits.shape
+    _check(temperature, "temperature", F32, (r,))
+    _check(u, "u", F32, (r,))
+    _check(tokens, "tokens", I32, (r,))
+    if top_k is not None:
+        _check(top_k, "top_k", I32, (r,))
+    if top_p is not None:
+        _check(top_p, "top_p", F32, (r,))
+    f = _fn("sampling", "kvf_sample", [c_void_p, c_int, c_int, c_int] + [c_void_p] * 6)
+    _ok(f(logits.data_ptr(), logits.stride(0) if r > 1 else v, r, v, temperature.data_ptr(),
+          top_k.data_ptr() if top_k is not None else None,
+          top_p.data_ptr() if top_p is not None else None, u.data_ptr(), tokens.data_ptr(),
+          _stream()), "sample")

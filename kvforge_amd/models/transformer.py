@@ -1,0 +1,106 @@
+"""The runnable model: a ``ModelSpec`` (parts chosen by the registry's builder) with its weights
+on the device, its cache groups worked out, and one ``forward`` over a flat batch
+(src/tokenvault/model.py:175-191)."""
+
+from __future__ import annotations
+
+import torch
+
+from kvforge_amd import registry
+from kvforge_amd.cache.manager import CacheGroup
+from kvforge_amd.kernels import library
+from kvforge_amd.parts.base import CacheSpec, LayerState, ModelSpec, StateSpec
+from kvforge_amd.weights.loader import load_model_weights
+
+
+class Transformer:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device: torch.device | str) -> None:
+        self.spec, self.config = spec, spec.config
+        self.dtype, self.device = dtype, device
+        self.order = spec.run_order()
+        n = len(spec.blocks)
+        for c in self.order:
+            if not 0 <= c.layer < n or (c.cache_of is not None and not 0 <= c.cache_of < n):
+                raise ValueError(f"run order names a layer outside 0..{n - 1}: {c}")
+        # blocks that own pages: those some call runs with its own cache
+        owners = sorted({c.layer for c in self.order if c.cache_of is None
+                         and spec.blocks[c.layer].mixer.cache_spec is not None})
+        for c in self.order:
+            if c.cache_of is not None and c.cache_of not in owners:
+                raise ValueError(f"layer {c.layer} reads the cache of layer {c.cache_of}, "
+                                 "which owns none")
+        by_spec: dict[CacheSpec, list[int]] = {}
+        for i in owners:
+            by_spec.setdefault(spec.blocks[i].mixer.cache_spec, []).append(i)
+        self.cache_groups = [CacheGroup(tuple(layers), cs.num_kv_heads, cs.head_dim, cs.window)
+                             for cs, layers in by_spec.items()]
+        self.state_specs: dict[int, StateSpec] = {
+            i: b.mixer.state_spec for i, b in enumerate(spec.blocks) if b.mixer.state_spec is not None}
+        self.layer_states: list[LayerState] = []
+        self._loaded = False
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, folder: str, dtype: torch.dtype, device: torch.device | str = "cuda"
+                    ) -> "Transformer":
+        cfg = registry.config_from_folder(folder)
+        model = cls(registry.build_spec(cfg), dtype, device)
+        model.load_folder(folder)
+        return model
+
+    def load_folder(self, folder: str) -> None:
+        load_model_weights(self.spec, folder, self.dtype, self.device)
+        self._loaded = True
+
+    def kernel_modules(self) -> list[str]:
+        mods: set[str] = {"elementwise", "sampling"}
+        for p in self.spec.all_parts():
+            mods |= p.kernel_modules(self.dtype)
+        return sorted(m for m in mods if m in library.available_modules())
+
+    def prepare(self, max_positions: int) -> None:
+        for p in self.spec.positions:
+            p.prepare(max_positions, self.device)
+
+    def attach(self, storage, states) -> None:
+        """Bind every call of the run order to its pages and state tensor."""
+        self.layer_states = []
+        for c in self.order:
+            src = c.layer if c.cache_of is None else c.cache_of
+            ls = LayerState(owns_cache=c.cache_of is None)
+            if src in storage.k:
+                ls.group, ls.k_pages, ls.v_pages = storage.group_of[src], storage.k[src], storage.v[src]
+            if states is not None and c.layer in states.tensors:
+                ls.state = states.tensors[c.layer]
+            self.layer_states.append(ls)
+
+    @property
+    def weight_bytes(self) -> int:
+        seen: dict[int, int] = {}
+        for p in self.spec.all_parts():
+            for t in vars(p).values():
+                if isinstance(t, torch.Tensor) and t.is_floating_point() and t.dim() >= 1:
+                    seen[t.data_ptr()] = t.numel() * t.element_size()
+        return sum(seen.values())
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, step) -> torch.Tensor:
+        """Runs the step's tokens from the cache; returns fp32 logits ``[n_logits, vocab]`` (a
+        view of workspace memory, valid until the next forward)."""
+        spec = self.spec
+        cfg = self.config
+        hidden = spec.embedding.hidden
+        residual = step.ws.buf("residual", (step.n_tokens, hidden), torch.float32)
+        spec.embedding.forward(step.token_ids, residual)
+        for p in spec.positions:
+            p.on_embedding(residual, step)
+        for call, ls in zip(self.order, self.layer_states):
+            spec.blocks[call.layer].forward(residual, step, ls)
+        r = step.n_logits
+        if r == 0:
+            return torch.empty((0, cfg.vocab_size), dtype=torch.float32, device=residual.device)
+        x = step.ws.buf("final_normed", (r, hidden), step.act_dtype)
+        spec.final_norm.forward(residual, x, step.logits_rows)
+        logits = step.ws.buf("logits", (r, cfg.vocab_size), torch.float32)
+        spec.head.forward(x, logits)
+        return logits

@@ -1,0 +1,94 @@
+"""Grouped-query causal attention over the paged cache (src/tokenvault/model.py:64-92).
+
+Order of work per call, as in the reference: project q, k, v; rotate q and k; write k and v into
+the cache; attend from the cache (the current tokens' keys are read back from it); project out.
+Query runs longer than one token go to the prefill kernel, single tokens to the decode kernel;
+both read the same pages through the same block tables.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from kvforge_amd.kernels import ops
+from kvforge_amd.parts.base import CacheSpec, LayerState, Mixer, WeightSpec
+from kvforge_amd.parts.positions import RotaryPositions
+from kvforge_amd.registry import register_mixer
+
+
+@register_mixer("attention")
+class PagedAttention(Mixer):
+    """``window``: ``None`` attends to every earlier position, ``w`` to the last ``w``."""
+
+    def __init__(self, prefix: str, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 rotary: RotaryPositions | None, scale: float | None = None,
+                 window: int | None = None) -> None:
+        if num_heads % num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(
+                f"attention kernels take head sizes in steps of 16 up to 256, got {head_dim}")
+        self.prefix = prefix
+        self.hidden, self.H, self.KV, self.d = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.rotary = rotary
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.window = int(window) if window else None
+        self.cache_spec = CacheSpec(self.KV, self.d, self.window)
+        self.w_qkv: torch.Tensor | None = None
+        self.w_o: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, H, KV, d = self.hidden, self.H, self.KV, self.d
+        return {
+            self._name("q_proj.weight"): WeightSpec((H * d, h)),
+            self._name("k_proj.weight"): WeightSpec((KV * d, h)),
+            self._name("v_proj.weight"): WeightSpec((KV * d, h)),
+            self._name("o_proj.weight"): WeightSpec((h, H * d)),
+        }
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        q, k, v = (tensors[self._name(f"{n}_proj.weight")] for n in "qkv")
+        if not (q.dtype == k.dtype == v.dtype):
+            q, k, v = q.float(), k.float(), v.float()
+        # one product for the three projections: rows of q heads, then k heads, then v heads
+        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
+        self.w_o = tensors[self._name("o_proj.weight")]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        mods = {"elementwise", "gemm_generic", "attn_generic", "attn_decode"}
+        if dtype == torch.bfloat16:
+            mods |= {"gemm_bf16"}
+        return mods
+
+    def num_bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in (self.w_qkv, self.w_o) if t is not None)
+
+    def forward(self, x, step, layer: LayerState, residual) -> None:
+        n = x.shape[0]
+        H, KV, d = self.H, self.KV, self.d
+        ws = step.ws
+        qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), x.dtype)
+        ops.gemm(x, self.w_qkv, qkv)
+        table = step.block_tables[layer.group]
+        if self.rotary is not None:
+            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, self.rotary.cos,
+                             self.rotary.sin, table, layer.k_pages, layer.v_pages, H, KV, d,
+                             write_kv=layer.owns_cache)
+        else:
+            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, step.unit_cos(),
+                             step.zero_sin(), table, layer.k_pages, layer.v_pages, H, KV, d,
+                             write_kv=layer.owns_cache)
+        out = ws.buf("attn_out", (n, H * d), x.dtype)
+        window = self.window or 0
+        work = step.prefill_work(H // KV)
+        if work is not None:
+            ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
+                             work, out, H, KV, d, self.scale, window)
+        if step.n_decode:
+            splits, workspace = step.decode_plan(H, KV, d, window)
+            ops.attn_decode(qkv, layer.k_pages, layer.v_pages, table, step.decode_seq_ids,
+                            step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
+                            window, splits, workspace)
+        ops.gemm(out, self.w_o, residual, accumulate=True)

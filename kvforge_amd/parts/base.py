@@ -1,0 +1,192 @@
+"""What every part of a model is made of.
+
+A *part* (norm, position encoding, mixer, feed-forward, embedding, head) takes its sizes and
+constants as constructor arguments, names the checkpoint tensors it needs, and knows nothing of
+the model it sits in.  A *block* arranges parts around the fp32 residual stream.  A model is a
+list of blocks plus the order in which they run (``LayerCall``), which is data: a block may be
+named twice, and a call may use another block's cache.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import TYPE_CHECKING
+
+import torch
+
+if TYPE_CHECKING:  # pragma: no cover
+    from kvforge_amd.engine.batch import Step
+
+
+@dataclass(frozen=True)
+class WeightSpec:
+    """One checkpoint tensor a part expects.
+
+    ``init`` drives the random-weights mode: ``"normal"`` draws N(0, std), ``"norm"`` draws
+    1 + N(0, std), ``"zeros"`` is zero.  ``integer`` tensors are tables of int32."""
+
+    shape: tuple[int, ...]
+    init: str = "normal"
+    std: float = 0.02
+    integer: bool = False
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """A mixer's need for keys and values that grow with the sequence.
+
+    ``window``: ``None`` keeps every position; ``w`` keeps the last ``w`` positions, and pages
+    wholly behind the window are given back while the request is live.  Layers with equal specs
+    form one cache group with pages and block tables of its own."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """A mixer's per-request state of fixed size: one slot of ``shape`` per live request."""
+
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerState:
+    """What a mixer call is handed besides activations: the cache pages it reads and writes
+    (possibly another block's), the group whose block tables address them, and its state slots."""
+
+    group: int | None = None
+    k_pages: torch.Tensor | None = None
+    v_pages: torch.Tensor | None = None
+    owns_cache: bool = True
+    state: torch.Tensor | None = None
+
+
+class Part:
+    """Base of all parts.  ``prefix`` is the part's place in the checkpoint's name space."""
+
+    prefix: str = ""
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        """Take the named tensors (already on the device, already in their run-time dtype)."""
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return set()
+
+    def num_bytes(self) -> int:
+        """Bytes of weights this part reads in one step."""
+        return 0
+
+    def _name(self, local: str) -> str:
+        return f"{self.prefix}.{local}" if self.prefix else local
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+        """``out[m] = norm(x[rows[m] or m])``; ``x`` is the fp32 residual stream."""
+        raise NotImplementedError
+
+
+class Positions(Part):
+    """Position encoding.  Two hooks, both optional: one on the embedding output (absolute
+    encodings) and tables a mixer applies to queries and keys (rotary encodings)."""
+
+    def prepare(self, max_positions: int, device: torch.device | str) -> None:
+        """Build per-position tables for positions ``0..max_positions-1``."""
+
+    def on_embedding(self, residual: torch.Tensor, step: "Step") -> None:
+        """Modify the embedding output in place (default: nothing)."""
+
+
+class Mixer(Part):
+    """Mixes information across the tokens of a sequence (attention, recurrences, ...)."""
+
+    cache_spec: CacheSpec | None = None
+    state_spec: StateSpec | None = None
+
+    def forward(self, x: torch.Tensor, step: "Step", layer: LayerState,
+                residual: torch.Tensor) -> None:
+        """Add the mixer's output for activations ``x [N, hidden]`` into ``residual`` (fp32)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, step: "Step", residual: torch.Tensor) -> None:
+        """Add the feed-forward output for ``x [N, hidden]`` into ``residual`` (fp32)."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of parts around the residual stream."""
+
+    mixer: Mixer
+
+    def parts(self) -> list[Part]:
+        raise NotImplementedError
+
+    def forward(self, residual: torch.Tensor, step: "Step", layer: LayerState) -> None:
+        raise NotImplementedError
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        out: dict[str, WeightSpec] = {}
+        for p in self.parts():
+            out.update(p.weight_specs())
+        return out
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        for p in self.parts():
+            p.load(tensors)
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        out: set[str] = set()
+        for p in self.parts():
+            out |= p.kernel_modules(dtype)
+        return out
+
+    def num_bytes(self) -> int:
+        return sum(p.num_bytes() for p in self.parts())
+
+
+@dataclass(frozen=True)
+class LayerCall:
+    """One entry of the run order: run block ``layer``; ``cache_of`` names the block whose cache
+    it uses (``None``: its own, which it also writes)."""
+
+    layer: int
+    cache_of: int | None = None
+
+
+@dataclass
+class ModelSpec:
+    """Everything the registry's builder decides for one architecture."""
+
+    config: object
+    embedding: Part
+    blocks: list[Block]
+    final_norm: Norm
+    head: Part
+    positions: list[Positions] = field(default_factory=list)
+    schedule: list[LayerCall] | None = None
+    # checkpoint names that may be present and are not loaded (regular expressions)
+    ignored_weights: tuple[str, ...] = ()
+
+    def run_order(self) -> list[LayerCall]:
+        return self.schedule if self.schedule is not None else [
+            LayerCall(i) for i in range(len(self.blocks))]
+
+    def all_parts(self) -> list[Part]:
+        return [self.embedding, *self.positions, *self.blocks, self.final_norm, self.head]
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        out: dict[str, WeightSpec] = {}
+        for p in self.all_parts():
+            for name, spec in p.weight_specs().items():
+                if name in out and out[name] != spec:
+                    raise ValueError(f"two parts expect {name} with different shapes")
+                out[name] = spec
+        return out

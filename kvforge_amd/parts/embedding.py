@@ -1,0 +1,54 @@
+"""Token embedding and the output head (src/tokenvault/model.py:153-158,169-170,190-191)."""
+
+from __future__ import annotations
+
+import torch
+
+from kvforge_amd.kernels import ops
+from kvforge_amd.parts.base import Part, WeightSpec
+
+
+class TokenEmbedding(Part):
+    """``h0 = table[ids]`` into the fp32 residual stream; no scaling."""
+
+    def __init__(self, prefix: str, vocab: int, hidden: int) -> None:
+        self.prefix, self.vocab, self.hidden = prefix, int(vocab), int(hidden)
+        self.table: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self._name("weight"): WeightSpec((self.vocab, self.hidden))}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.table = tensors[self._name("weight")]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return {"elementwise"}
+
+    def forward(self, ids: torch.Tensor, out: torch.Tensor) -> None:
+        ops.embed(ids, self.table, out)
+
+
+class LMHead(Part):
+    """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
+    table when the head shares it (then no tensor of its own is expected)."""
+
+    def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None) -> None:
+        self.prefix, self.vocab, self.hidden, self.tied_to = prefix, int(vocab), int(hidden), tied_to
+        self.weight: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        if self.tied_to is not None:
+            return {self.tied_to: WeightSpec((self.vocab, self.hidden))}
+        return {self._name("weight"): WeightSpec((self.vocab, self.hidden))}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.tied_to if self.tied_to is not None else self._name("weight")]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return {"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
+
+    def num_bytes(self) -> int:
+        return self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
+
+    def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
+        ops.gemm(x, self.weight, logits)

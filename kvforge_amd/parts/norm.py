@@ -1,0 +1,33 @@
+"""RMS norm over the fp32 residual stream (src/tokenvault/model.py:28-38)."""
+
+from __future__ import annotations
+
+import torch
+
+from kvforge_amd.kernels import ops
+from kvforge_amd.parts.base import Norm, WeightSpec
+from kvforge_amd.registry import register_norm
+
+
+@register_norm("rmsnorm")
+class RMSNorm(Norm):
+    """``y = x * rsqrt(mean(x^2) + eps) * weight`` in fp32, rounded once to the output type."""
+
+    def __init__(self, prefix: str, width: int, eps: float) -> None:
+        self.prefix, self.width, self.eps = prefix, int(width), float(eps)
+        self.weight: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self._name("weight"): WeightSpec((self.width,), init="norm", std=0.1)}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.weight = tensors[self._name("weight")]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return {"elementwise"}
+
+    def num_bytes(self) -> int:
+        return self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+        ops.rmsnorm(x, self.weight, self.eps, out, rows)

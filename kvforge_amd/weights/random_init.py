@@ -1,0 +1,49 @@
+"""Random-weights mode: writes a model folder (``config.json``, ``model.safetensors``) from a
+configuration and a seed.
+
+The reference's ``build_model`` (src/tokenvault/model_loader.py:42-61) draws every matrix from
+N(0, 0.02) under one seed and sets norm weights to a constant.  Here norm weights are drawn from
+1 + N(0, 0.1), because a kernel that forgets a constant-one weight still passes, and the tensors
+go through the same files and loader as a real checkpoint.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from kvforge_amd import registry
+from kvforge_amd.weights.io import write_safetensors
+
+_STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.Tensor]:
+    """Tensors for every name the model expects, drawn in sorted name order from one generator."""
+    store = _STORE[dtype]
+    gen = torch.Generator().manual_seed(int(seed))
+    out: dict[str, torch.Tensor] = {}
+    for name, w in sorted(spec.weight_specs().items()):
+        if w.integer:
+            out[name] = torch.zeros(w.shape, dtype=torch.int32)
+        elif w.init == "zeros":
+            out[name] = torch.zeros(w.shape, dtype=store)
+        else:
+            t = torch.randn(w.shape, generator=gen, dtype=torch.float32) * w.std
+            if w.init == "norm":
+                t = t + 1.0
+            elif w.init != "normal":
+                raise ValueError(f"unknown init {w.init!r} for {name}")
+            out[name] = t.to(store)
+    return out
+
+
+def write_random_model(folder: str, config: "dict[str, Any] | Any", seed: int = 0,
+                       dtype: str = "bfloat16") -> str:
+    """``config``: a config.json dictionary or a typed configuration."""
+    cfg = registry.config_from_dict(config) if isinstance(config, dict) else config
+    spec = registry.build_spec(cfg)
+    cfg.save(folder)
+    write_safetensors(folder, random_tensors(spec, seed, dtype))
+    return folder

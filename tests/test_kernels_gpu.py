@@ -1,0 +1,360 @@
+"""Each HIP kernel alone against a plain fp32 torch reference, at sizes other than the engine's
+(odd widths, head sizes that are no power of two, group sizes 1/3/4/6, scattered pages)."""
+
+from __future__ import annotations
+
+import math
+import random
+
+import pytest
+import torch
+
+from tests.plain import llama as plain
+from tests.plain import sampling as plain_sampling
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def ops():
+    from kvforge_amd.kernels import ops as o
+    return o
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(37, 48, generator=g).to(dtype)
+    ids = torch.tensor([0, 36, 5, 5, 99, -1, 17], dtype=torch.int32)
+    out = torch.full((7, 48), 7.0, device=DEV)
+    ops().embed(ids.to(DEV), table.to(DEV), out)
+    want = torch.zeros(7, 48)
+    for i, t in enumerate(ids.tolist()):
+        if 0 <= t < 37:
+            want[i] = table[t].float()
+    assert torch.equal(out.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h", [96, 100, 2048, 3000])
+@pytest.mark.parametrize("w32", [False, True])
+def test_rmsnorm(dtype, h, w32):
+    g = torch.Generator().manual_seed(h)
+    x = torch.randn(9, h, generator=g) * 3
+    w = (1 + 0.1 * torch.randn(h, generator=g))
+    w = w if w32 else w.to(dtype)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    out = torch.empty(4, h, dtype=dtype, device=DEV)
+    ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-5, out, rows.to(DEV))
+    want = plain.rms_norm(x[rows.long()], w.float(), 1e-5)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    # against the library routine
+    lib = torch.nn.functional.rms_norm(x[rows.long()], (h,), w.float(), 1e-5)
+    torch.testing.assert_close(out.float().cpu(), lib, **tol(dtype))
+    out2 = torch.empty(9, h, dtype=dtype, device=DEV)
+    ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-6, out2)
+    torch.testing.assert_close(out2.float().cpu(), plain.rms_norm(x, w.float(), 1e-6), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    g = torch.Generator().manual_seed(1)
+    gu = (torch.randn(5, 2 * 176, generator=g) * 2).to(dtype)
+    out = torch.empty(5, 176, dtype=dtype, device=DEV)
+    ops().silu_mul(gu.to(DEV), out)
+    want = torch.nn.functional.silu(gu[:, :176].float()) * gu[:, 176:].float()
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("ta", DTYPES)
+@pytest.mark.parametrize("tw", DTYPES)
+@pytest.mark.parametrize("mnk", [(1, 384, 96), (5, 37, 50), (70, 130, 96), (33, 256, 176),
+                                 (130, 70, 257)])
+def test_gemm_generic(ta, tw, mnk):
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(m * n + k)
+    a = torch.randn(m, k, generator=g).to(ta)
+    w = (torch.randn(n, k, generator=g) * 0.1).to(tw)
+    want = a.double() @ w.double().T
+    for out_dtype in DTYPES:
+        out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+        ops().gemm(a.to(DEV), w.to(DEV), out)
+        t = tol(out_dtype)
+        torch.testing.assert_close(out.double().cpu(), want, **t)
+    res = torch.randn(m, n, generator=g)
+    acc = res.clone().to(DEV)
+    ops().gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
+    torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=2e-5, rtol=2e-5)
+    # a view with a wider row stride
+    wide = torch.zeros(m, k + 24, dtype=ta)
+    wide[:, :k] = a
+    out = torch.empty(m, n, dtype=torch.float32, device=DEV)
+    ops().gemm(wide.to(DEV)[:, :k], w.to(DEV), out)
+    torch.testing.assert_close(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
+
+
+def test_gemm_rows_do_not_depend_on_batch():
+    """fp32 products are accumulated in one fixed order: a row alone equals the row in a batch."""
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(77, 176, generator=g).to(DEV)
+    w = torch.randn(300, 176, generator=g).to(DEV)
+    full = torch.empty(77, 300, device=DEV)
+    ops().gemm(a, w, full)
+    one = torch.empty(1, 300, device=DEV)
+    ops().gemm(a[40:41], w, one)
+    assert torch.equal(one[0], full[40])
+
+
+class Paged:
+    """Scatters contiguous per-sequence K/V into shuffled pages ``[nb, KV, bs, d]``."""
+
+    def __init__(self, seq_lens, KV, d, bs, dtype, seed=0, spare=7):
+        rng = random.Random(seed)
+        g = torch.Generator().manual_seed(seed)
+        need = sum(-(-n // bs) for n in seq_lens)
+        self.nb = need + spare
+        ids = list(range(self.nb))
+        rng.shuffle(ids)
+        self.k = torch.randn(self.nb, KV, bs, d, generator=g).to(dtype)  # junk everywhere
+        self.v = torch.randn(self.nb, KV, bs, d, generator=g).to(dtype)
+        width = max(-(-n // bs) for n in seq_lens) + 2
+        self.table = torch.full((len(seq_lens), width), -1, dtype=torch.int32)
+        self.keys, self.values = [], []
+        for s, n in enumerate(seq_lens):
+            kk = torch.randn(n, KV, d, generator=g).to(dtype)
+            vv = torch.randn(n, KV, d, generator=g).to(dtype)
+            for b in range(-(-n // bs)):
+                page = ids.pop()
+                self.table[s, b] = page
+                seg = slice(b * bs, min(n, (b + 1) * bs))
+                cnt = seg.stop - seg.start
+                self.k[page, :, :cnt] = kk[seg].transpose(0, 1)
+                self.v[page, :, :cnt] = vv[seg].transpose(0, 1)
+            self.keys.append(kk)
+            self.values.append(vv)
+
+
+def attn_reference(paged, q, seq_lens, q_lens, scale, window):
+    outs, off = [], 0
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        outs.append(plain.causal_attention(q[off:off + ql].float(), paged.keys[s].float(),
+                                           paged.values[s].float(), scale, n - ql, window))
+        off += ql
+    return torch.cat(outs)
+
+
+def prefill_work(q_lens, G):
+    work = []
+    for s, ql in enumerate(q_lens):
+        for t in range(-(-ql * G // 16)):
+            work.append((s, t))
+    return torch.tensor(work, dtype=torch.int32).reshape(-1, 2)
+
+
+# the (context, query) cases of the reference's tests/test_paged_attention.py:60-66 and more
+ATTN_CASES = [
+    ([9, 16], [9, 16]),
+    ([12, 30, 5], [4, 7, 5]),
+    ([17, 3, 25], [2, 3, 5]),
+    ([200, 131], [67, 131]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seq_lens,q_lens", ATTN_CASES)
+@pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
+                                        (4, 4, 80, 16), (8, 2, 128, 16), (2, 1, 256, 32)])
+@pytest.mark.parametrize("window", [0, 11])
+def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
+    paged = Paged(seq_lens, KV, d, bs, dtype, seed=len(seq_lens) + d)
+    g = torch.Generator().manual_seed(d)
+    n = sum(q_lens)
+    # q lives inside a wider qkv-like buffer
+    buf = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    q = buf[:, :H * d].reshape(n, H, d)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    ctx = torch.tensor(seq_lens, dtype=torch.int32)
+    out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
+    scale = 1 / math.sqrt(d)
+    ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                       cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV).to(DEV), out,
+                       H, KV, d, scale, window)
+    want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
+                                        (4, 4, 80, 16), (32, 8, 64, 16), (8, 2, 128, 16),
+                                        (12, 1, 112, 16), (2, 1, 256, 32)])
+@pytest.mark.parametrize("splits", [1, 3])
+@pytest.mark.parametrize("window", [0, 11])
+def test_attn_decode(dtype, H, KV, d, bs, splits, window):
+    seq_lens = [7, 13, 1, 20, 300, 64]  # tests/test_paged_attention.py:61 of the reference + long
+    q_lens = [1] * len(seq_lens)
+    paged = Paged(seq_lens, KV, d, bs, dtype, seed=d + H)
+    g = torch.Generator().manual_seed(d)
+    n = len(seq_lens)
+    buf = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    q = buf[:, :H * d].reshape(n, H, d)
+    cu = torch.arange(n + 1, dtype=torch.int32)
+    ctx = torch.tensor(seq_lens, dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
+    ws = (torch.empty(n * H * splits * d, device=DEV), torch.empty(n * H * splits * 2, device=DEV))
+    out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
+    ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, n,
+                      cu.to(DEV), ctx.to(DEV), out, H, KV, d, scale, window, splits, ws)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    # a subset of the sequences, named by seq_ids; the others stay untouched
+    ids = torch.tensor([4, 1], dtype=torch.int32)
+    out2 = torch.full((n, H * d), 5.0, dtype=dtype, device=DEV)
+    ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                      ids.to(DEV), 2, cu.to(DEV), ctx.to(DEV), out2, H, KV, d, scale, window,
+                      splits, ws)
+    got = out2.float().cpu()
+    torch.testing.assert_close(got[[4, 1]], want[[4, 1]], **tol(dtype))
+    assert (got[[0, 2, 3, 5]] == 5.0).all()
+
+
+def test_attn_far_key_stands_out():
+    """One key among hundreds carries the weight: q and that key are scaled so that its score
+    dominates; a kernel that drops or misplaces a page shows at once."""
+    H, KV, d, bs = 4, 2, 64, 16
+    for far in (0, 15, 16, 255, 256, 511):
+        seq_lens = [600]
+        paged = Paged(seq_lens, KV, d, bs, torch.float32, seed=far)
+        g = torch.Generator().manual_seed(far)
+        q = torch.randn(1, H, d, generator=g)
+        for kvh in range(KV):
+            key = paged.keys[0][far, kvh]
+            for gi in range(H // KV):
+                q[0, kvh * (H // KV) + gi] = key * 40.0 / key.norm() ** 2 * math.sqrt(d)
+        buf = torch.zeros(1, (H + 2 * KV) * d)
+        buf[:, :H * d] = q.reshape(1, -1)
+        cu = torch.tensor([0, 1], dtype=torch.int32)
+        ctx = torch.tensor(seq_lens, dtype=torch.int32)
+        want = attn_reference(paged, q, seq_lens, [1], 1 / math.sqrt(d), None).reshape(1, H * d)
+        # the far key's value dominates
+        assert (want.reshape(H, d)[0] - paged.values[0][far, 0]).abs().max() < 0.05
+        for splits in (1, 4):
+            ws = (torch.empty(H * splits * d, device=DEV), torch.empty(H * splits * 2, device=DEV))
+            out = torch.zeros(1, H * d, device=DEV)
+            ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                              None, 1, cu.to(DEV), ctx.to(DEV), out, H, KV, d, 1 / math.sqrt(d), 0,
+                              splits, ws)
+            torch.testing.assert_close(out.cpu(), want, atol=2e-5, rtol=2e-5)
+        out = torch.zeros(1, H * d, device=DEV)
+        ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                           cu.to(DEV), ctx.to(DEV), prefill_work([1], H // KV).to(DEV), out,
+                           H, KV, d, 1 / math.sqrt(d), 0)
+        torch.testing.assert_close(out.cpu(), want, atol=2e-5, rtol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16)])
+def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
+    g = torch.Generator().manual_seed(d)
+    seq_lens = [5, 19]
+    starts = [2, 0]                      # the first sequence already holds two tokens
+    n = sum(seq_lens)
+    qkv = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    positions = torch.tensor([starts[0] + i for i in range(5)] + list(range(19)), dtype=torch.int32)
+    seq_of = torch.tensor([0] * 5 + [1] * 19, dtype=torch.int32)
+    nb = 12
+    table = torch.tensor([[7, 3, -1, -1, -1], [1, 9, 4, 0, 2]], dtype=torch.int32)[:, : -(-21 // bs) + 1]
+    table = table.contiguous()
+    inv_freq = plain.rope_inv_freq(rot, 10000.0)
+    cos_full, sin_full = plain.rope_cos_sin(torch.arange(40), inv_freq)
+    cos_t, sin_t = cos_full[:, : rot // 2].contiguous(), sin_full[:, : rot // 2].contiguous()
+    kp = torch.zeros(nb, KV, bs, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(nb, KV, bs, d, dtype=dtype, device=DEV)
+    dev_qkv = qkv.to(DEV).clone()
+    ops().rope_kvwrite(dev_qkv, positions.to(DEV), seq_of.to(DEV), cos_t.to(DEV), sin_t.to(DEV),
+                       table.to(DEV), kp, vp, H, KV, d)
+    cos, sin = plain.rope_cos_sin(positions, inv_freq)
+    qf = qkv[:, :H * d].float().reshape(n, H, d)
+    kf = qkv[:, H * d:(H + KV) * d].float().reshape(n, KV, d)
+    vf = qkv[:, (H + KV) * d:].float().reshape(n, KV, d)
+
+    def rot_part(x):
+        r = plain.apply_rope(x[..., :rot], cos, sin)
+        return torch.cat([r, x[..., rot:]], -1)
+
+    want_q, want_k = rot_part(qf), rot_part(kf)
+    got_q = dev_qkv[:, :H * d].float().cpu().reshape(n, H, d)
+    torch.testing.assert_close(got_q, want_q, **tol(dtype))
+    kp, vp = kp.float().cpu(), vp.float().cpu()
+    for t in range(n):
+        s, p = int(seq_of[t]), int(positions[t])
+        page, off = int(table[s, p // bs]), p % bs
+        if page < 0:
+            continue
+        torch.testing.assert_close(kp[page, :, off], want_k[t], **tol(dtype))
+        torch.testing.assert_close(vp[page, :, off], vf[t], **tol(dtype))
+    # nothing else was written
+    written = torch.zeros(nb, bs, dtype=torch.bool)
+    for t in range(n):
+        s, p = int(seq_of[t]), int(positions[t])
+        if int(table[s, p // bs]) >= 0:
+            written[int(table[s, p // bs]), p % bs] = True
+    assert (kp.abs().sum((1, 3))[~written] == 0).all()
+
+
+def test_sample_greedy_and_filters():
+    # src/tokenvault tests/test_continuous_batching.py:160-169: logits [4,3,2,1,0]
+    logits = torch.tensor([[4.0, 3.0, 2.0, 1.0, 0.0]] * 4, device=DEV)
+    temp = torch.tensor([0.0, 1.0, 1.0, 1.0], device=DEV)
+    top_k = torch.tensor([0, 2, 0, 1], dtype=torch.int32, device=DEV)
+    top_p = torch.tensor([1.0, 1.0, 0.5, 1.0], device=DEV)
+    toks = torch.empty(4, dtype=torch.int32, device=DEV)
+    for u in (0.0, 0.3, 0.72, 0.74, 0.999):
+        uu = torch.full((4,), u, device=DEV)
+        ops().sample(logits, temp, top_k, top_p, uu, toks)
+        got = toks.tolist()
+        assert got[0] == 0
+        p2 = plain_sampling.processed_probs(logits[1].cpu(), 1.0, top_k=2)
+        assert got[1] == plain_sampling.draw(p2, u) and got[1] in (0, 1)
+        assert got[2] == 0          # top_p = 0.5 keeps only the first (mass 0.64)
+        assert got[3] == 0
+
+
+@pytest.mark.parametrize("V", [384, 5000, 128256])
+def test_sample_matches_plain(V):
+    g = torch.Generator().manual_seed(V)
+    rows = 12
+    logits = torch.randn(rows, V, generator=g) * 3
+    temps = [0.0, 0.8, 1.0, 0.5, 1.3, 0.8, 0.8, 1.0, 0.7, 2.0, 0.0, 1.0]
+    ks = [0, 0, 50, 0, 7, 20, 0, 1, 0, 0, 5, 300]
+    ps = [1.0, 1.0, 1.0, 0.9, 0.8, 1.0, 0.3, 1.0, 0.95, 1.0, 0.5, 0.6]
+    us = [plain_sampling.uniform(V, r, 3) for r in range(rows)]
+    toks = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops().sample(logits.to(DEV), torch.tensor(temps, device=DEV),
+                 torch.tensor(ks, dtype=torch.int32, device=DEV), torch.tensor(ps, device=DEV),
+                 torch.tensor(us, device=DEV), toks)
+    got = toks.tolist()
+    for r in range(rows):
+        probs = plain_sampling.processed_probs(logits[r], temps[r], ks[r], ps[r])
+        if temps[r] == 0.0:
+            assert got[r] == int(logits[r].argmax())
+            continue
+        assert probs[got[r]] > 0, f"row {r}: token {got[r]} was filtered out"
+        # equal to the plain draw unless u falls within rounding of an interval's edge
+        assert plain_sampling.draw_margin(probs, us[r], got[r]) < 1e-5, f"row {r}"
+
+
+def test_sample_frequencies_follow_softmax():
+    logits = torch.tensor([1.0, 0.0, -1.0, 2.0, 0.5])
+    n = 4000
+    us = torch.tensor([plain_sampling.uniform(7, 0, i) for i in range(n)])
+    toks = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops().sample(logits.repeat(n, 1).to(DEV), torch.full((n,), 0.8, device=DEV), None, None,
+                 us.to(DEV), toks)
+    freq = torch.bincount(toks.cpu().long(), minlength=5).double() / n
+    want = torch.softmax(logits.double() / 0.8, -1)
+    assert (freq - want).abs().max() < 0.03
