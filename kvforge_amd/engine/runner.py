@@ -78,3 +78,12 @@ class ModelRunner:
         self.num_forward_passes += 1
         self.num_tokens_processed += step.n_tokens
         return logits
+
+    @torch.inference_mode()
+    def step_and_sample(self, entries: Sequence[StepEntry], sampler, params, streams, counters
+                        ) -> list[int]:
+        """One forward, then one token for every wanted place (in row order)."""
+        logits = self.step(entries)
+        if logits.shape[0] != len(params):
+            raise ValueError("one SamplingParams per wanted place")
+        return sampler(logits, params, streams, counters)
