@@ -1,0 +1,81 @@
+"""The batch builder on the CPU: the exact arrays of the reference's
+tests/test_continuous_batching.py:27-39, padding, and what is refused."""
+
+from __future__ import annotations
+
+import pytest
+import torch
+
+from kvforge_amd.cache import CacheGroup, CacheManager
+from kvforge_amd.engine.batch import MetaBuffers, Step, StepEntry, Workspace, fill_step
+
+
+def setup(num_blocks=16, bs=4, groups=None):
+    groups = groups or [CacheGroup((0,), 1, 16, None)]
+    cache = CacheManager(bs, groups, num_blocks)
+    meta = MetaBuffers(64, 8, [8] * len(groups), "cpu")
+    step = Step()
+    step.ws, step.device = Workspace("cpu"), "cpu"
+    return cache, meta, step
+
+
+def test_flat_varlen_batch_reference_vector():
+    cache, meta, step = setup()
+    cache.allocate("a", 6)
+    cache.allocate("b", 2)
+    counts = fill_step(step, meta, [StepEntry("a", [1, 2, 3], 3, "last"), StepEntry("b", [9], 1, "all")],
+                       cache.block_table, lambda r: -1, 4)
+    assert step.token_ids.tolist() == [1, 2, 3, 9]
+    assert step.positions.tolist() == [3, 4, 5, 1]
+    assert step.cu_q.tolist() == [0, 3, 4]
+    assert step.ctx_lens.tolist() == [6, 2]
+    assert step.logits_rows.tolist() == [2, 3] and counts == [1, 1]
+    assert step.seq_of_token.tolist() == [0, 0, 0, 1]
+    ta, tb = cache.block_table("a"), cache.block_table("b")
+    assert step.block_tables[0][0, :2].tolist() == ta and step.block_tables[0][1, :1].tolist() == tb
+    assert (step.block_tables[0][0, 2:] == -1).all()
+    # a slot computed as the kernels do equals the manager's
+    for tok in range(4):
+        s, p = int(step.seq_of_token[tok]), int(step.positions[tok])
+        slot = int(step.block_tables[0][s, p // 4]) * 4 + p % 4
+        assert slot == cache.slot("ab"[s], p)
+    assert step.n_decode == 1 and step.decode_seq_ids.tolist() == [1] and step.prefill_seqs == [0]
+    assert step.prefill_work(2).tolist() == [[0, 0]] and step.prefill_work(6).tolist() == [[0, 0], [0, 1]]
+
+
+def test_wanted_places_and_modes():
+    cache, meta, step = setup()
+    cache.allocate("a", 8)
+    cache.allocate("b", 2)
+    counts = fill_step(step, meta, [StepEntry("a", [5, 6, 7, 8], 0, [0, 2]),
+                                    StepEntry("b", [1, 2], 0, "none")],
+                       cache.block_table, lambda r: -1, 4)
+    assert step.logits_rows.tolist() == [0, 2] and counts == [2, 0]
+    with pytest.raises(ValueError):
+        StepEntry("a", [1], 0, [1]).wanted()
+    with pytest.raises(ValueError):
+        StepEntry("a", [1], 0, "some").wanted()
+
+
+def test_pure_decode_padding_is_inert():
+    cache, meta, step = setup()
+    for r in "ab":
+        cache.allocate(r, 5)
+    fill_step(step, meta, [StepEntry("a", [3], 4), StepEntry("b", [4], 4)], cache.block_table,
+              lambda r: -1, 4, pad_to=4)
+    assert step.n_seqs == 4 and step.n_tokens == 4 and step.n_decode == 4
+    assert step.decode_seq_ids is None
+    assert step.ctx_lens.tolist() == [5, 5, 0, 0]
+    assert (step.block_tables[0][2:] == -1).all()
+    assert step.max_decode_ctx == 5 and step.n_logits == 2
+
+
+def test_refusals():
+    cache, meta, step = setup()
+    cache.allocate("a", 4)
+    with pytest.raises(ValueError, match="pages"):
+        fill_step(step, meta, [StepEntry("a", [1, 2], 4)], cache.block_table, lambda r: -1, 4)
+    with pytest.raises(ValueError, match="capacity"):
+        fill_step(step, meta, [StepEntry("a", [1] * 65, 0)], cache.block_table, lambda r: -1, 4)
+    with pytest.raises(ValueError):
+        fill_step(step, meta, [], cache.block_table, lambda r: -1, 4)

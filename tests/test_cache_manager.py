@@ -1,0 +1,199 @@
+"""The cache manager alone: the reference's allocator vectors (tests/test_block_manager.py of the
+reference), windows, state slots, and random orders of requests under which no page may be lost,
+held twice or freed twice."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+
+from kvforge_amd.cache import (RELEASED, BlockPool, CacheGroup, CacheManager, NoFreeBlocksError,
+                               StateSlots)
+
+FULL = CacheGroup(layers=(0, 1), num_kv_heads=2, head_dim=16, window=None)
+
+
+def mgr(num_blocks, block_size, groups=(FULL,), **kw):
+    return CacheManager(block_size, list(groups), num_blocks, **kw)
+
+
+def test_allocate_and_free_roundtrip():           # reference tests/test_block_manager.py:6-13
+    m = mgr(8, 4)
+    m.allocate("a", 10)
+    assert len(m.block_table("a")) == 3 and m.num_free_blocks == 5
+    m.free("a")
+    assert m.num_free_blocks == 8
+
+
+def test_slot_mapping_is_block_major():            # :16-22
+    m = mgr(8, 4)
+    m.allocate("a", 6)
+    t = m.block_table("a")
+    assert m.slot("a", 0) == t[0] * 4 and m.slot("a", 5) == t[1] * 4 + 1
+    assert t == [0, 1]                             # page 0 is handed out first
+
+
+def test_growth_only_at_block_boundary():          # :25-31
+    m = mgr(8, 4)
+    m.allocate("a", 3)
+    m.append_slots("a", 4, 3)
+    assert len(m.block_table("a")) == 1
+    m.append_slots("a", 5, 4)
+    assert len(m.block_table("a")) == 2
+
+
+def test_exhaustion_is_detected():                 # :34-40
+    m = mgr(2, 4)
+    m.allocate("a", 8)
+    assert not m.can_allocate(1) and not m.can_append_slots("a", 9, 8)
+    with pytest.raises(NoFreeBlocksError):
+        m.allocate("b", 1)
+    with pytest.raises(NoFreeBlocksError):
+        m.append_slots("a", 9, 8)
+    assert m.num_free_blocks == 0 and len(m.block_table("a")) == 2   # nothing half-taken
+
+
+def test_free_unknown_is_a_noop_and_double_release_raises():   # :70-75
+    m = mgr(4, 4)
+    m.allocate("a", 2)
+    m.free("a")
+    m.free("a")
+    assert m.num_free_blocks == 4
+    pool = BlockPool(2)
+    b = pool.take()
+    pool.release(b)
+    with pytest.raises(RuntimeError, match="double free"):
+        pool.release(b)
+    m.allocate("b", 1)
+    with pytest.raises(ValueError):
+        m.allocate("b", 1)
+
+
+def test_fragmentation_stats():                    # :119-125
+    m = mgr(16, 8)
+    m.allocate("a", 9)
+    s = m.stats()
+    assert s.num_used_blocks == 2
+    assert s.internal_fragmentation == pytest.approx(1 - 9 / 16)
+    assert s.utilization == pytest.approx(2 / 16)
+
+
+def test_watermark_holds_back_admission_only():
+    m = mgr(10, 4, watermark=0.2)                  # 2 pages kept free at admission
+    assert m.can_allocate(32) and not m.can_allocate(33)
+    m.allocate("a", 32)
+    assert m.can_append_slots("a", 40, 32)         # growth may use the reserve
+
+
+def test_lifo_reuse():
+    m = mgr(4, 4)
+    m.allocate("a", 8)
+    m.allocate("b", 4)
+    ta = list(m.block_table("a"))
+    m.free("a")
+    m.allocate("c", 8)
+    assert sorted(m.block_table("c")) == sorted(ta)       # the pages just freed are used again
+
+
+def test_window_group_gives_pages_back_early():
+    win = CacheGroup(layers=(1,), num_kv_heads=1, head_dim=16, window=6)
+    m = mgr(8, 4, groups=(CacheGroup((0,), 1, 16, None), win))
+    m.allocate("a", 0)
+    m.append_slots("a", 10, 0)
+    assert len(m.block_table("a", 0)) == 3 and len(m.block_table("a", 1)) == 3
+    # after 10 tokens the next query (position 10) sees keys from 5 on: page 0 (0..3) is behind
+    assert m.release_behind("a", 10) == 1
+    assert m.block_table("a", 1)[0] == RELEASED and m.block_table("a", 0)[0] != RELEASED
+    assert m.pools[1].num_free == 6 and m.pools[0].num_free == 5
+    # growing never takes a released page back
+    m.append_slots("a", 17, 10)
+    assert m.block_table("a", 1)[0] == RELEASED and len(m.block_table("a", 1)) == 5
+    m.release_behind("a", 17)                      # sees from 12: pages 0..2 are behind
+    assert m.block_table("a", 1)[:3] == [RELEASED] * 3
+    m.free("a")
+    assert m.pools[0].num_free == 8 and m.pools[1].num_free == 8
+
+
+def test_window_group_needs_fewer_pages_for_later_portions():
+    win = CacheGroup(layers=(0,), num_kv_heads=1, head_dim=16, window=4)
+    m = mgr(3, 4, groups=(win,))
+    m.allocate("a", 0)
+    m.append_slots("a", 8, 0)                      # two pages
+    m.release_behind("a", 8)                       # sees from 5: page 0 goes back
+    assert m.can_append_slots("a", 16, 8)          # needs pages 2, 3: two free
+    m.append_slots("a", 16, 8)
+    assert m.num_free_blocks == 0
+
+
+def test_state_slots():
+    s = StateSlots(2)
+    a, b = s.take("a"), s.take("b")
+    assert {a, b} == {0, 1} and s.num_free == 0
+    with pytest.raises(NoFreeBlocksError):
+        s.take("c")
+    with pytest.raises(ValueError):
+        s.take("a")
+    s.release("a")
+    s.release("a")
+    assert s.take("c") == a
+    m = mgr(8, 4, num_state_slots=1)
+    m.allocate("x", 4)
+    assert m.slots.slot("x") == 0 and not m.can_allocate(1)
+    m.free("x")
+    assert m.can_allocate(1) and m.slots.num_free == 1
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_lose_nothing(seed):
+    """Requests arrive, grow, pass windows and end in random order: every page is either free or
+    held by exactly one table entry, counts agree, and at the end everything is free."""
+    rng = random.Random(seed)
+    bs = rng.choice([4, 8, 16])
+    groups = (CacheGroup((0, 2), 2, 16, None), CacheGroup((1,), 1, 32, rng.choice([5, 16, 40])))
+    counts = [rng.randint(8, 24), rng.randint(8, 24)]
+    m = CacheManager(bs, list(groups), counts, num_state_slots=5)
+    live: dict[str, int] = {}
+
+    def check():
+        for g, pool in enumerate(m.pools):
+            held = [b for rid in live for b in m.block_table(rid, g) if b != RELEASED]
+            assert len(held) == len(set(held)), "a page is held twice"
+            assert len(held) + pool.num_free == pool.num_blocks, "a page was lost"
+            assert all(pool.ref_count(b) == 1 for b in held)
+            assert not set(held) & set(pool._free)
+        assert m.slots.num_free == 5 - len(live)
+
+    n = 0
+    for _ in range(400):
+        op = rng.random()
+        if op < 0.3 and len(live) < 5:
+            rid, toks = f"r{n}", rng.randint(1, 3 * bs)
+            n += 1
+            if m.can_allocate(toks):
+                m.allocate(rid, toks)
+                live[rid] = toks
+                m.release_behind(rid, toks)
+            else:
+                with pytest.raises(NoFreeBlocksError):
+                    m.allocate(rid, toks)
+        elif op < 0.8 and live:
+            rid = rng.choice(list(live))
+            total = live[rid] + rng.randint(1, 2 * bs)
+            if m.can_append_slots(rid, total, live[rid]):
+                m.append_slots(rid, total, live[rid])
+                live[rid] = total
+                m.release_behind(rid, total)
+            else:
+                with pytest.raises(NoFreeBlocksError):
+                    m.append_slots(rid, total, live[rid])
+        elif live:
+            rid = rng.choice(list(live))
+            m.free(rid)
+            del live[rid]
+        check()
+    for rid in list(live):
+        m.free(rid)
+    live.clear()
+    check()
+    assert all(p.num_free == p.num_blocks for p in m.pools)
