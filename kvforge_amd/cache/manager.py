@@ -20,8 +20,8 @@ RELEASED = -1  # table entry of a page that was given back (or never held)
 
 @dataclass(frozen=True)
 class CacheGroup:
-    """Layers whose mixers have equal cache needs.  ``layers``: indices of the blocks that own
-    pages in this group."""
+    """Layers whose mixers have equal cache needs.  ``layers``: places in the model's run order
+    of the calls that own pages in this group."""
 
     layers: tuple[int, ...]
     num_kv_heads: int

@@ -18,24 +18,33 @@ class Transformer:
         self.spec, self.config = spec, spec.config
         self.dtype, self.device = dtype, device
         self.order = spec.run_order()
-        n = len(spec.blocks)
+        n, calls = len(spec.blocks), len(self.order)
         for c in self.order:
-            if not 0 <= c.layer < n or (c.cache_of is not None and not 0 <= c.cache_of < n):
+            if not 0 <= c.layer < n:
                 raise ValueError(f"run order names a layer outside 0..{n - 1}: {c}")
-        # blocks that own pages: those some call runs with its own cache
-        owners = sorted({c.layer for c in self.order if c.cache_of is None
-                         and spec.blocks[c.layer].mixer.cache_spec is not None})
-        for c in self.order:
-            if c.cache_of is not None and c.cache_of not in owners:
-                raise ValueError(f"layer {c.layer} reads the cache of layer {c.cache_of}, "
-                                 "which owns none")
+        # Pages and state belong to a *call* (an entry of the run order), not to a block: a block
+        # named twice shares its weights, and each of its calls keeps a cache of its own.
+        owners = [i for i, c in enumerate(self.order) if c.cache_of is None
+                  and spec.blocks[c.layer].mixer.cache_spec is not None]
+        for i, c in enumerate(self.order):
+            if c.cache_of is None:
+                continue
+            if not 0 <= c.cache_of < calls or c.cache_of not in owners:
+                raise ValueError(f"call {i} reads the cache of call {c.cache_of}, which owns none")
+            if c.cache_of >= i:
+                raise ValueError(f"call {i} reads the cache of a later call ({c.cache_of})")
+            a = spec.blocks[c.layer].mixer.cache_spec
+            b = spec.blocks[self.order[c.cache_of].layer].mixer.cache_spec
+            if a != b:
+                raise ValueError(f"call {i} and call {c.cache_of} need different caches: {a} / {b}")
         by_spec: dict[CacheSpec, list[int]] = {}
         for i in owners:
-            by_spec.setdefault(spec.blocks[i].mixer.cache_spec, []).append(i)
-        self.cache_groups = [CacheGroup(tuple(layers), cs.num_kv_heads, cs.head_dim, cs.window)
-                             for cs, layers in by_spec.items()]
+            by_spec.setdefault(spec.blocks[self.order[i].layer].mixer.cache_spec, []).append(i)
+        self.cache_groups = [CacheGroup(tuple(ix), cs.num_kv_heads, cs.head_dim, cs.window)
+                             for cs, ix in by_spec.items()]
         self.state_specs: dict[int, StateSpec] = {
-            i: b.mixer.state_spec for i, b in enumerate(spec.blocks) if b.mixer.state_spec is not None}
+            i: spec.blocks[c.layer].mixer.state_spec for i, c in enumerate(self.order)
+            if spec.blocks[c.layer].mixer.state_spec is not None}
         self.layer_states: list[LayerState] = []
         self._loaded = False
 
@@ -65,13 +74,13 @@ class Transformer:
     def attach(self, storage, states) -> None:
         """Bind every call of the run order to its pages and state tensor."""
         self.layer_states = []
-        for c in self.order:
-            src = c.layer if c.cache_of is None else c.cache_of
+        for i, c in enumerate(self.order):
+            src = i if c.cache_of is None else c.cache_of
             ls = LayerState(owns_cache=c.cache_of is None)
             if src in storage.k:
                 ls.group, ls.k_pages, ls.v_pages = storage.group_of[src], storage.k[src], storage.v[src]
-            if states is not None and c.layer in states.tensors:
-                ls.state = states.tensors[c.layer]
+            if states is not None and i in states.tensors:
+                ls.state = states.tensors[i]
             self.layer_states.append(ls)
 
     @property

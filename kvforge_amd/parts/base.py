@@ -154,8 +154,9 @@ class Block(Part):
 
 @dataclass(frozen=True)
 class LayerCall:
-    """One entry of the run order: run block ``layer``; ``cache_of`` names the block whose cache
-    it uses (``None``: its own, which it also writes)."""
+    """One entry of the run order: run block ``layer``.  ``cache_of``: ``None`` gives the call a
+    cache of its own, which it writes and reads; an index into the run order (of an earlier
+    call) makes it read that call's cache and write none."""
 
     layer: int
     cache_of: int | None = None

@@ -1,0 +1,292 @@
+"""Generation through the entry point (``InferenceEngine.generate`` / ``step``) against the plain
+model: the reference's end-to-end tests (tests/test_continuous_batching.py:42-169 of the
+reference) on this engine, plus sampling that does not depend on batching."""
+
+from __future__ import annotations
+
+import random
+
+import pytest
+import torch
+
+import kvforge_amd
+from kvforge_amd import (CacheConfig, EngineConfig, InferenceEngine, RequestStatus, SamplingParams,
+                         SchedulerConfig)
+from tests.plain import llama as plain
+from tests.plain import sampling as plain_sampling
+
+pytestmark = pytest.mark.gpu
+GREEDY = SamplingParams(max_tokens=10, temperature=0.0)
+
+
+class Oracle:
+    """Plain greedy continuation that also reports how safe each choice was."""
+
+    def __init__(self, folder):
+        self.w = kvforge_amd.read_safetensors_folder(folder)
+        self.cfg = plain.read_config(folder)
+
+    def greedy(self, prompt, n):
+        ids, out, gaps = list(prompt), [], []
+        for _ in range(n):
+            logits = plain.forward(self.w, self.cfg, ids)[-1]
+            top = torch.topk(logits, 2).values
+            gaps.append(float(top[0] - top[1]))
+            out.append(int(logits.argmax()))
+            ids.append(out[-1])
+        return out, gaps
+
+    def logits(self, ids):
+        return plain.forward(self.w, self.cfg, ids)
+
+    def check_choices(self, prompt, out, margin):
+        """Every generated token is the plain model's argmax, given the engine's own history, up
+        to ``margin`` in the logits (one plain forward covers all places, by causality)."""
+        logits = self.logits(list(prompt) + list(out))
+        for i, tok in enumerate(out):
+            row = logits[len(prompt) - 1 + i]
+            assert float(row.max() - row[tok]) <= margin, (
+                f"token {i} = {tok}: plain logit {row[tok]:.5f}, best {row.max():.5f} "
+                f"at {int(row.argmax())}")
+
+
+def assert_greedy_equal(got, want, gaps, margin=1e-4):
+    """Tokens must agree up to the first place where the plain model's top two logits are closer
+    than ``margin`` (there rounding may choose either and the continuations part ways)."""
+    for i, (g, w, gap) in enumerate(zip(got, want, gaps)):
+        if gap < margin:
+            return
+        assert g == w, f"token {i}: engine {g}, plain {w} (gap {gap:.2e}); got {got}, want {want}"
+    assert len(got) == len(want)
+
+
+@pytest.fixture(scope="module")
+def model_a(tmp_path_factory):
+    folder = str(tmp_path_factory.mktemp("tiny_a"))
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-a"), seed=0)
+    return folder, Oracle(folder)
+
+
+@pytest.fixture(scope="module")
+def model_b(tmp_path_factory):
+    folder = str(tmp_path_factory.mktemp("tiny_b"))
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1)
+    return folder, Oracle(folder)
+
+
+def engine_for(folder, dtype="float32", block_size=4, num_blocks=256, max_num_seqs=8,
+               max_num_batched_tokens=256, **kw):
+    cfg = EngineConfig(cache=CacheConfig(block_size=block_size, num_blocks=num_blocks),
+                       scheduler=SchedulerConfig(max_num_seqs=max_num_seqs,
+                                                 max_num_batched_tokens=max_num_batched_tokens),
+                       dtype=dtype, **kw)
+    return InferenceEngine.from_folder(folder, cfg)
+
+
+def prompts_for(vocab, n, seed, lo=2, hi=30):
+    rng = random.Random(seed)
+    return [[rng.randrange(1, vocab) for _ in range(rng.randint(lo, hi))] for _ in range(n)]
+
+
+def test_baseline_config_a(model_a):
+    """Tiny Llama A, fp32, seed 0, block 16: prompts of 5/17/33 tokens, greedy, 16 new each."""
+    folder, oracle = model_a
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, 256, (n,), generator=g).tolist() for n in (5, 17, 33)]
+    engine = engine_for(folder, block_size=16, num_blocks=64)
+    outs = engine.generate(prompts, SamplingParams(max_tokens=16, temperature=0.0))
+    for p, o in zip(prompts, outs):
+        want, gaps = oracle.greedy(p, 16)
+        assert_greedy_equal(o.output_token_ids, want, gaps)
+        assert o.finish_reason.value == "length" and o.prompt_token_ids == p
+
+
+def test_baseline_config_b_chunked_temperature(model_b):
+    """Tiny Llama B, fp32, seed 1, block 8: prompts of 1/9/40/70 tokens, chunk 24 mixed with
+    decodes, temperature 0.8, 12 new.  Every sampled token must be the plain rule's draw from the
+    plain model's logits of the engine's own token history."""
+    folder, oracle = model_b
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, 384, (n,), generator=g).tolist() for n in (1, 9, 40, 70)]
+    engine = engine_for(folder, block_size=8, num_blocks=64, max_num_batched_tokens=24, seed=1)
+    params = SamplingParams(max_tokens=12, temperature=0.8)
+    outs = engine.generate(prompts, params)
+    assert max(engine.metrics.batch_sizes) >= 2 and max(engine.metrics.batched_tokens) <= 24
+    for stream, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o.output_token_ids) == 12
+        logits = oracle.logits(p + o.output_token_ids)
+        for i, tok in enumerate(o.output_token_ids):
+            probs = plain_sampling.processed_probs(logits[len(p) - 1 + i], 0.8)
+            u = plain_sampling.uniform(1, stream, i)
+            assert plain_sampling.draw_margin(probs, u, tok) < 1e-4, (stream, i, tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_batched_output_equals_isolated_greedy(model_a, dtype):
+    folder, oracle = model_a
+    prompts = prompts_for(256, 6, 0)
+    engine = engine_for(folder, dtype)
+    outs = engine.generate(prompts, GREEDY)
+    for p, o in zip(prompts, outs):
+        assert len(o.output_token_ids) == 10
+        if dtype == "float32":
+            want, gaps = oracle.greedy(p, 10)
+            assert min(gaps) > 1e-4
+            assert o.output_token_ids == want
+        else:
+            oracle.check_choices(p, o.output_token_ids, 3e-2)
+
+
+def test_requests_join_running_batch(model_a):
+    folder, oracle = model_a
+    prompts = prompts_for(256, 4, 1)
+    engine = engine_for(folder)
+    engine.add_request(prompts[0], GREEDY, request_id="r0")
+    engine.add_request(prompts[1], GREEDY, request_id="r1")
+    done, step = {}, 0
+    while engine.has_unfinished_requests():
+        if step == 3:
+            engine.add_request(prompts[2], GREEDY, request_id="r2")
+        if step == 5:
+            engine.add_request(prompts[3], GREEDY, request_id="r3")
+        if step == 4:
+            assert engine.scheduler.num_running == 3
+        for out in engine.step():
+            if out.finished:
+                done[out.request_id] = out.output_token_ids
+        step += 1
+    for i, p in enumerate(prompts):
+        want, gaps = oracle.greedy(p, 10)
+        assert_greedy_equal(done[f"r{i}"], want, gaps)
+    assert max(engine.metrics.batch_sizes) >= 3
+
+
+def test_short_requests_leave_early_and_free_pages(model_a):
+    folder, _ = model_a
+    engine = engine_for(folder)
+    engine.add_request([1, 2, 3], SamplingParams(max_tokens=2, temperature=0), request_id="short")
+    engine.add_request([4, 5, 6], SamplingParams(max_tokens=12, temperature=0), request_id="long")
+    finished_at, step = {}, 0
+    while engine.has_unfinished_requests():
+        for o in engine.step():
+            if o.finished:
+                finished_at[o.request_id] = step
+        step += 1
+    assert finished_at["short"] < finished_at["long"]
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
+def test_pages_run_out_preemption_preserves_outputs(model_a):
+    folder, oracle = model_a
+    prompts = prompts_for(256, 6, 2)
+    engine = engine_for(folder, num_blocks=14, max_num_seqs=6, max_num_batched_tokens=64)
+    outs = engine.generate(prompts, GREEDY)
+    assert engine.scheduler.num_preemptions > 0
+    for p, o in zip(prompts, outs):
+        want, gaps = oracle.greedy(p, 10)
+        assert_greedy_equal(o.output_token_ids, want, gaps)
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
+@pytest.mark.parametrize("budget", [16, 24])
+def test_chunked_prefill_preserves_outputs(model_a, budget):
+    folder, oracle = model_a
+    prompts = [list(range(1, 60)), list(range(100, 140))]
+    engine = engine_for(folder, max_num_batched_tokens=budget)
+    outs = engine.generate(prompts, GREEDY)
+    assert max(engine.metrics.batched_tokens) <= budget
+    for p, o in zip(prompts, outs):
+        want, gaps = oracle.greedy(p, 10)
+        assert_greedy_equal(o.output_token_ids, want, gaps)
+
+
+def test_abort_mid_generation(model_a):
+    folder, _ = model_a
+    engine = engine_for(folder)
+    rid = engine.add_request([1, 2, 3], SamplingParams(max_tokens=50))
+    engine.step()
+    engine.step()
+    req = engine.scheduler.requests[rid]
+    assert req.status == RequestStatus.RUNNING
+    assert engine.abort_request(rid)
+    assert req.status == RequestStatus.ABORTED and not engine.has_unfinished_requests()
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+    assert not engine.abort_request(rid)
+
+
+def test_stop_token_and_metrics(model_a):
+    folder, oracle = model_a
+    want, _ = oracle.greedy([7, 7, 7], 10)
+    stop = want[3]
+    engine = engine_for(folder)
+    out = engine.generate([[7, 7, 7]], SamplingParams(max_tokens=10, temperature=0,
+                                                      stop_token_ids=[stop]))[0]
+    assert out.output_token_ids == want[: want.index(stop) + 1]
+    assert out.finish_reason.value == "stop"
+    stats = engine.stats()
+    m = stats["metrics"]
+    assert m["requests_finished"] == 1 and m["output_tokens_per_s"] > 0 and m["ttft_p50_ms"] > 0
+    assert stats["forward_passes"] == engine.runner.num_forward_passes > 0
+    assert stats["kv_cache"]["num_free_blocks"] == stats["kv_cache"]["num_blocks"]
+    assert stats["weights_bytes"] > 0
+
+
+def test_sampling_does_not_depend_on_batching(model_b):
+    """The same request, alone and inside a busy chunked batch, draws the same tokens: the
+    uniform numbers are keyed by (seed, request stream, output index), not by batch order."""
+    folder, _ = model_b
+    target = list(range(3, 40))
+    params = SamplingParams(max_tokens=12, temperature=0.8, top_k=50, top_p=0.9, seed=77)
+    alone = engine_for(folder, block_size=8, seed=5).generate([target], params)[0].output_token_ids
+    others = prompts_for(384, 5, 9, 10, 60)
+    busy = engine_for(folder, block_size=8, seed=5, max_num_batched_tokens=24)
+    outs = busy.generate(others[:3] + [target] + others[3:],
+                         [SamplingParams(max_tokens=9, temperature=1.0)] * 3 + [params]
+                         + [SamplingParams(max_tokens=20, temperature=0.0)] * 2)
+    assert outs[3].output_token_ids == alone
+    again = engine_for(folder, block_size=8, seed=5).generate([target], params)[0].output_token_ids
+    other_seed = engine_for(folder, block_size=8, seed=6).generate([target], params)[0].output_token_ids
+    assert again == alone and other_seed != alone
+
+
+def test_rejections_at_the_entry_point(model_a):
+    folder, _ = model_a
+    engine = engine_for(folder)
+    with pytest.raises(ValueError, match="vocabulary"):
+        engine.add_request([1, 999])
+    with pytest.raises(ValueError, match="tokenizer"):
+        engine.add_request("text")
+    with pytest.raises(ValueError):
+        engine.add_request([])
+    with pytest.raises(ValueError, match="max_model_len"):
+        engine.add_request(list(range(128)))     # max_position_embeddings of tiny-a
+
+
+def test_long_decoding(model_b):
+    """200 tokens decoded from a short prompt in bfloat16 and float32 stay on the plain model's
+    greedy path wherever that path is safe."""
+    folder, oracle = model_b
+    prompt = [11, 45, 200, 3]
+    want, gaps = oracle.greedy(prompt, 200)
+    for dtype, margin in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        engine = engine_for(folder, dtype, block_size=8)
+        out = engine.generate([prompt], SamplingParams(max_tokens=200, temperature=0.0))[0]
+        assert len(out.output_token_ids) == 200
+        oracle.check_choices(prompt, out.output_token_ids, margin)
+        if dtype == "float32":
+            assert_greedy_equal(out.output_token_ids, want, gaps, margin)
+
+
+def test_command_line(model_a, capsys):
+    from kvforge_amd import generate
+    folder, oracle = model_a
+    rc = generate.main(["--model", folder, "--prompt-ids", "5,17,3", "--prompt-ids", "9 8 7 6",
+                        "--max-tokens", "6", "--temperature", "0", "--block-size", "4",
+                        "--num-blocks", "32", "--json"])
+    assert rc == 0
+    import json
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    for p, o in zip(([5, 17, 3], [9, 8, 7, 6]), rec["outputs"]):
+        want, gaps = oracle.greedy(p, 6)
+        assert_greedy_equal(o["output_token_ids"], want, gaps)
+    assert rec["stats"]["kv_cache"]["num_blocks"] == 32
