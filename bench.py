@@ -1,0 +1,186 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512]
+                    [--dtype bfloat16] [--layers L] [--no-points]
+
+Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
+size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
+N(0, 0.02), batch 8, 512-token uniform-random prompts, greedy, context cap 8192, pages of 16
+tokens.  A step is one decode step of the whole engine (scheduler, batch building, forward,
+sampling, bookkeeping).  One JSON line is printed; besides the decode figure it carries a
+2,048-token prefill, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
+for fp32.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+CONTEXT_CAP = 8192
+BLOCK_SIZE = 16
+PREFILL_TOKENS = 2048
+
+
+def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True):
+    import kvforge_amd
+    from kvforge_amd import CacheConfig, EngineConfig, InferenceEngine, SchedulerConfig
+
+    num_blocks = -(-num_tokens_cached // BLOCK_SIZE) + max_num_seqs + 8
+    cfg = EngineConfig(
+        cache=CacheConfig(block_size=BLOCK_SIZE, num_blocks=num_blocks, watermark=0.0),
+        scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=PREFILL_TOKENS,
+                                  max_model_len=CONTEXT_CAP),
+        dtype=dtype, use_graphs=use_graphs)
+    return InferenceEngine.from_folder(folder, cfg)
+
+
+def random_prompts(vocab, n, length, seed):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(1, vocab, (length,), generator=g).tolist() for _ in range(n)]
+
+
+def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
+    """Prefill ``batch`` prompts, run ``warmup`` decode steps untimed, then time ``steps``."""
+    import torch
+    from kvforge_amd import SamplingParams
+
+    params = SamplingParams(max_tokens=steps + warmup + 8, temperature=0.0, ignore_eos=True)
+    for p in random_prompts(vocab, batch, prompt_len, seed):
+        engine.add_request(p, params)
+    while any(r.is_prefill for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    ctx_start = [r.num_tokens for r in engine.scheduler.running]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    produced = 0
+    for _ in range(steps):
+        produced += sum(len(o.new_token_ids) for o in engine.step())
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx_end = [r.num_tokens for r in engine.scheduler.running]
+    for rid in list(engine.scheduler.requests):
+        engine.abort_request(rid)
+    mean_ctx = (sum(ctx_start) + sum(ctx_end)) / 2.0 / max(1, batch)
+    return {"tokens": produced, "seconds": dt, "tok_s": produced / dt, "ms_per_step": dt / steps * 1e3,
+            "mean_ctx": mean_ctx}
+
+
+def prefill_run(engine, vocab, tokens, repeats=3, seed=1):
+    import torch
+    from kvforge_amd import SamplingParams
+
+    best = None
+    params = SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True)
+    for i in range(repeats + 1):
+        prompt = random_prompts(vocab, 1, tokens, seed + i)[0]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.generate([prompt], params)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i > 0:                      # the first run warms buffers and kernels
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def model_numbers(cfg, layers_run):
+    h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
+                         cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
+    per_layer = h * d * (2 * H + 2 * KV) + 3 * h * I
+    return {"linear_params": layers_run * per_layer, "head_params": V * h,
+            "kv_values_per_token": 2 * layers_run * KV * d, "attn_hd": H * d, "layers": layers_run}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=255)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
+    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-graphs", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
+        return 2
+
+    import torch
+    import kvforge_amd
+
+    cfg = kvforge_amd.preset_dict("llama-1b")
+    full_layers = cfg["num_hidden_layers"]
+    layers_run = args.layers or full_layers
+    cfg["num_hidden_layers"] = layers_run
+    elem = 2 if args.dtype == "bfloat16" else 4
+    nums = model_numbers(cfg, layers_run)
+    vocab = cfg["vocab_size"]
+
+    with tempfile.TemporaryDirectory(prefix="kvforge_bench_") as folder:
+        kvforge_amd.write_random_model(folder, cfg, seed=0)
+        results = {}
+        batches = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
+        for b in batches:
+            need = b * (args.prompt_len + args.steps + args.warmup + 16)
+            engine = build_engine(folder, args.dtype, max(b, 1), max(need, PREFILL_TOKENS + 64),
+                                  use_graphs=not args.no_graphs)
+            results[b] = decode_run(engine, vocab, b, args.prompt_len, args.steps, args.warmup)
+            if b == args.batch:
+                prefill_s = prefill_run(engine, vocab, PREFILL_TOKENS)
+                weight_bytes = engine.model.weight_bytes
+            del engine
+            torch.cuda.empty_cache()
+
+    main_run = results[args.batch]
+    step_s = main_run["seconds"] / args.steps
+    kv_bytes = args.batch * main_run["mean_ctx"] * nums["kv_values_per_token"] * elem
+    achieved = (weight_bytes + kv_bytes) / step_s / 1e9
+    n = PREFILL_TOKENS
+    prefill_flops = (2.0 * n * nums["linear_params"] + 2.0 * nums["head_params"]
+                     + 2.0 * n * n * nums["attn_hd"] * layers_run)
+    line = {
+        "metric": "decode tok/s (Llama 3.2 1B shape, batch %d)" % args.batch,
+        "value": round(main_run["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
+        "config": {
+            "model": "llama-3.2-1b-shape", "layers": full_layers, "layers_run": layers_run,
+            "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+            "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+            "intermediate": cfg["intermediate_size"], "vocab": vocab, "tied_embeddings": True,
+            "rope": "theta 5e5, llama3 factor 32", "rms_norm_eps": cfg["rms_norm_eps"],
+            "global_batch": args.batch, "seq_len": args.prompt_len, "new_tokens": args.steps + 1,
+            "context_len": CONTEXT_CAP, "block_size": BLOCK_SIZE, "parallelism": "single-gpu",
+            "sampling": "greedy",
+        },
+        "prefill": {"value": round(n / prefill_s, 1), "tokens": n, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_s / MFMA_PEAK[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -209,6 +209,11 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
         w = e.wanted()
         counts.append(len(w))
         rows.extend(int(cu[b]) + i for i in w)
+    if pad_to is not None:
+        # a padded batch has a fixed shape: one wanted row per sequence, padding included
+        if any(c != 1 for c in counts) or any(n != 1 for n in q_lens):
+            raise ValueError("padding is for batches of single tokens that each want their logits")
+        rows = list(range(Bp))
     R = len(rows)
     host[off["logits_rows"]:off["logits_rows"] + R] = rows
 

@@ -41,7 +41,8 @@ class InferenceEngine:
         sc, cc = config.scheduler, config.cache
         num_blocks = cc.resolve_num_blocks(ModelRunner.bytes_per_block(model, cc.block_size))
         self.runner = ModelRunner(model, cc.block_size, num_blocks, sc.max_num_seqs,
-                                  sc.max_num_batched_tokens, sc.max_model_len, cc.watermark)
+                                  sc.max_num_batched_tokens, sc.max_model_len, cc.watermark,
+                                  use_graphs=config.use_graphs)
         self.cache = self.runner.cache
         self.sampler = Sampler(config.seed, model.device)
         self.scheduler = Scheduler(sc, self.cache)

@@ -17,6 +17,8 @@ import torch
 from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
 from kvforge_amd.engine.batch import MetaBuffers, Step, StepEntry, Workspace, fill_step
+from kvforge_amd.kernels import ops
+from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
 from kvforge_amd.models.transformer import Transformer
 
@@ -24,7 +26,7 @@ from kvforge_amd.models.transformer import Transformer
 class ModelRunner:
     def __init__(self, model: Transformer, block_size: int, num_blocks: "int | list[int]",
                  max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
-                 watermark: float = 0.0) -> None:
+                 watermark: float = 0.0, use_graphs: bool = True) -> None:
         if torch.device(model.device).type != "cuda":
             raise RuntimeError("the engine runs on the GPU only; there is no CPU path")
         if not torch.cuda.is_available():
@@ -49,6 +51,15 @@ class ModelRunner:
         self.ws = Workspace(self.device)
         self.num_forward_passes = 0
         self.num_tokens_processed = 0
+        # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph
+        self.use_graphs = bool(use_graphs)
+        self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self.num_graph_replays = 0
+        cap = self.meta.max_seqs
+        self._sample_f = torch.zeros(3 * cap, dtype=torch.float32, device=self.device)
+        self._sample_i = torch.zeros(2 * cap, dtype=torch.int32, device=self.device)
+        self._sample_f_host = torch.zeros(3 * cap, dtype=torch.float32, pin_memory=True)
+        self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
 
     @staticmethod
     def bytes_per_block(model: Transformer, block_size: int) -> int:
@@ -83,7 +94,80 @@ class ModelRunner:
     def step_and_sample(self, entries: Sequence[StepEntry], sampler, params, streams, counters
                         ) -> list[int]:
         """One forward, then one token for every wanted place (in row order)."""
+        b = len(entries)
+        if (self.use_graphs and b == len(params) and b <= GRAPH_MAX_BATCH
+                and all(len(e.token_ids) == 1 and e.want == "last" for e in entries)):
+            return self._decode_step(entries, sampler.seed, params, streams, counters)
         logits = self.step(entries)
         if logits.shape[0] != len(params):
             raise ValueError("one SamplingParams per wanted place")
         return sampler(logits, params, streams, counters)
+
+    # ------------------------------------------------------------------ decode through graphs
+    def _decode_step(self, entries, seed, params, streams, counters) -> list[int]:
+        """A step of single tokens, padded to a bucket of batch sizes so that its launches can be
+        captured once in a HIP graph and replayed: metadata and sampling parameters live at fixed
+        device addresses and are refreshed by two copies before each replay."""
+        b = len(entries)
+        bucket = 1
+        while bucket < b:
+            bucket *= 2
+        bucket = min(bucket, self.meta.max_seqs)
+        step, _ = self.build_step(entries, pad_to=bucket)
+        ctx_bucket = 256
+        while ctx_bucket < step.max_decode_ctx:
+            ctx_bucket *= 2
+        step.max_decode_ctx = ctx_bucket
+        cap = self.meta.max_seqs
+        fh, ih = self._sample_f_host, self._sample_i_host
+        fh[:bucket] = 0.0                     # padding rows are greedy
+        fh[cap:cap + bucket] = 1.0
+        ih[:bucket] = 0
+        for i, (p, s, c) in enumerate(zip(params, streams, counters)):
+            fh[i] = p.temperature
+            fh[cap + i] = p.top_p
+            ih[i] = p.top_k
+            fh[2 * cap + i] = 0.0 if p.greedy else uniform(seed, s, c)
+        self._sample_f.copy_(fh, non_blocking=True)
+        self._sample_i[:cap].copy_(ih, non_blocking=True)
+        key = (bucket, ctx_bucket)
+        graph = self.graphs.get(key)
+        if graph is None:
+            self._forward_and_sample(step, bucket)          # the real result, and a warm-up
+            tokens = self._sample_i[cap:cap + b].tolist()
+            self.graphs[key] = self._capture(step, bucket)
+        else:
+            graph.graph.replay()
+            self.num_graph_replays += 1
+            tokens = self._sample_i[cap:cap + b].tolist()
+        self.num_forward_passes += 1
+        self.num_tokens_processed += b
+        return tokens
+
+    def _forward_and_sample(self, step: Step, rows: int) -> torch.Tensor:
+        cap = self.meta.max_seqs
+        logits = self.model.forward(step)
+        ops.sample(logits, self._sample_f[:rows], self._sample_i[:rows],
+                   self._sample_f[cap:cap + rows], self._sample_f[2 * cap:2 * cap + rows],
+                   self._sample_i[cap:cap + rows])
+        return logits
+
+    def _capture(self, step: Step, rows: int) -> "_DecodeGraph":
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        self.ws.frozen = True
+        try:
+            with torch.cuda.graph(graph):
+                logits = self._forward_and_sample(step, rows)
+        finally:
+            self.ws.frozen = False
+        # the graph keeps the workspace it was recorded with alive, whatever grows later
+        return _DecodeGraph(graph, logits, self.ws.snapshot())
+
+
+GRAPH_MAX_BATCH = 128  # beyond this the matrix products leave the weight-streaming kernel
+
+
+class _DecodeGraph:
+    def __init__(self, graph, logits, keep) -> None:
+        self.graph, self.logits, self.keep = graph, logits, keep

@@ -187,10 +187,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)
     if not accumulate:
         _tcode(out.dtype)
-    if a.dtype == BF16 and w.dtype == BF16 and _bf16_gemm_ok(m, n, k, lda, ldc):
-        f = _fn("gemm_bf16", "kvf_gemm_bf16", [c_void_p, c_void_p, c_void_p] + [c_int] * 6 + [c_void_p])
-        _ok(f(a.data_ptr(), w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc, _stream()),
-            "gemm_bf16")
+    if a.dtype == BF16 and w.dtype == BF16 and _bf16_gemm_ok(k, lda):
+        if m <= SKINNY_MAX_M or out_kind == 0:
+            f = _fn("gemm_bf16", "kvf_gemm_bf16",
+                    [c_void_p, c_void_p, c_void_p] + [c_int] * 6 + [c_void_p])
+            _ok(f(a.data_ptr(), w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc,
+                  _stream()), "gemm_bf16")
+        elif accumulate:
+            # many rows: the library's bf16 product (as the reference's engine uses one), then
+            # the residual sum in fp32
+            out.add_(torch.mm(a, w.t()))
+        else:
+            torch.mm(a, w.t(), out=out)
         return
     f = _fn("gemm_generic", "kvf_gemm_generic",
             [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_void_p])
@@ -198,10 +206,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
           m, n, k, lda, ldc, _stream()), "gemm_generic")
 
 
-def _bf16_gemm_ok(m: int, n: int, k: int, lda: int, ldc: int) -> bool:
-    """The MFMA kernels need K in steps of 32 and 16-byte aligned rows."""
-    return ("gemm_bf16" in library.available_modules() and k % 32 == 0 and lda % 8 == 0
-            and n % 16 == 0)
+def _bf16_gemm_ok(k: int, lda: int) -> bool:
+    """The MFMA kernel loads 16 bytes at a time: K and the row stride in steps of 8."""
+    return k % 8 == 0 and lda % 8 == 0
 
 
 # ------------------------------------------------------------------------------ attention

@@ -67,7 +67,12 @@ def test_pure_decode_padding_is_inert():
     assert step.decode_seq_ids is None
     assert step.ctx_lens.tolist() == [5, 5, 0, 0]
     assert (step.block_tables[0][2:] == -1).all()
-    assert step.max_decode_ctx == 5 and step.n_logits == 2
+    # a padded batch has a fixed shape: one logits row per sequence, padding included
+    assert step.max_decode_ctx == 5 and step.n_logits == 4
+    assert step.logits_rows.tolist() == [0, 1, 2, 3]
+    with pytest.raises(ValueError, match="padding"):
+        fill_step(step, meta, [StepEntry("a", [3], 4, "none")], cache.block_table, lambda r: -1, 4,
+                  pad_to=2)
 
 
 def test_refusals():

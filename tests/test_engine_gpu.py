@@ -290,3 +290,39 @@ def test_command_line(model_a, capsys):
         want, gaps = oracle.greedy(p, 6)
         assert_greedy_equal(o["output_token_ids"], want, gaps)
     assert rec["stats"]["kv_cache"]["num_blocks"] == 32
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager_steps(model_b, dtype):
+    """Decode steps replayed from captured HIP graphs give the tokens of the same steps launched
+    one kernel at a time: requests join and leave (the padded batch size and the context bucket
+    change, so several graphs are captured and each is replayed many times, with eager prefill
+    steps and synchronisations in between)."""
+    folder, _ = model_b
+    prompts = prompts_for(384, 7, 3, 3, 50)
+    params = [SamplingParams(max_tokens=n, temperature=t, top_k=k, top_p=p)
+              for n, t, k, p in ((40, 0.0, 0, 1.0), (25, 0.8, 0, 1.0), (60, 1.0, 40, 0.9),
+                                 (12, 0.0, 0, 1.0), (33, 0.7, 0, 0.8), (50, 0.0, 0, 1.0),
+                                 (45, 1.2, 10, 1.0))]
+
+    def run(use_graphs):
+        engine = engine_for(folder, dtype, block_size=8, max_num_seqs=5, max_num_batched_tokens=32,
+                            seed=11, use_graphs=use_graphs)
+        done, step = {}, 0
+        pending = list(zip(prompts, params))
+        for p, sp in pending[:3]:
+            engine.add_request(p, sp)
+        pending = pending[3:]
+        while engine.has_unfinished_requests() or pending:
+            if pending and step % 9 == 4:
+                engine.add_request(*pending.pop(0))
+            for o in engine.step():
+                if o.finished:
+                    done[o.request_id] = o.output_token_ids
+            step += 1
+        return done, engine
+
+    eager, _ = run(False)
+    graphed, engine = run(True)
+    assert len(engine.runner.graphs) >= 3 and engine.runner.num_graph_replays > 50
+    assert graphed == eager

@@ -98,6 +98,45 @@ def test_gemm_generic(ta, tw, mnk):
     torch.testing.assert_close(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64, 100, 128, 200, 300])
+@pytest.mark.parametrize("n,k", [(16, 40), (37, 96), (384, 176), (2048, 2048), (200, 8192), (3072, 64)])
+def test_gemm_bf16_mfma(m, n, k):
+    """bf16 x bf16 on the matrix cores: fp32 store, bf16 store and fp32 accumulate, with tails in
+    M, N and K."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    want = a.double() @ w.double().T
+    out = torch.empty(m, n, device=DEV)
+    ops().gemm(a.to(DEV), w.to(DEV), out)
+    torch.testing.assert_close(out.double().cpu(), want, atol=1e-4, rtol=1e-4)
+    outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops().gemm(a.to(DEV), w.to(DEV), outb)
+    torch.testing.assert_close(outb.double().cpu(), want, atol=2e-2, rtol=2e-2)
+    res = torch.randn(m, n, generator=g)
+    acc = res.clone().to(DEV)
+    ops().gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
+    t = dict(atol=1e-4, rtol=1e-4) if m <= 128 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(acc.double().cpu(), res.double() + want, **t)
+    # a strided view of a wider buffer as left operand
+    wide = torch.zeros(m, k + 16, dtype=torch.bfloat16)
+    wide[:, 8:k + 8] = a
+    out2 = torch.empty(m, n, device=DEV)
+    ops().gemm(wide.to(DEV)[:, 8:k + 8], w.to(DEV), out2)
+    torch.testing.assert_close(out2.double().cpu(), want, atol=1e-4, rtol=1e-4)
+
+
+def test_gemm_bf16_rows_do_not_depend_on_neighbours():
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(16, 2048, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(512, 2048, generator=g) / 45).to(torch.bfloat16).to(DEV)
+    full = torch.empty(16, 512, device=DEV)
+    ops().gemm(a, w, full)
+    one = torch.empty(1, 512, device=DEV)
+    ops().gemm(a[7:8], w, one)
+    assert torch.equal(one[0], full[7])
+
+
 def test_gemm_rows_do_not_depend_on_batch():
     """fp32 products are accumulated in one fixed order: a row alone equals the row in a batch."""
     g = torch.Generator().manual_seed(3)
