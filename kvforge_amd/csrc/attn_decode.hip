@@ -7,8 +7,9 @@
 // 64 / LPK keys per iteration and the four waves of a workgroup take consecutive key groups.
 // Every lane group keeps its own running maximum, sum and accumulator (fp32), rescaling only
 // when the maximum grows; groups, waves and splits are merged at the end with the usual
-// log-sum-exp rule.  With one split the output is written directly, otherwise partial
-// (max, sum, accumulator) triples go to a workspace that `kvf_attn_decode_combine` merges.
+// log-sum-exp rule.  With one split the output is written directly; otherwise partial
+// (max, sum, accumulator) triples go to a workspace and the workgroup that finishes last for a
+// (sequence, head chunk), found by a ticket counter, merges them in split order.
 //
 // A window w > 0 restricts the keys to (p - w, p].  Pages are [num_blocks, KV, block_size, d].
 #include "common.h"
@@ -30,10 +31,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, const int* __restrict__ seq_ids,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, T* __restrict__ out,
-    float* __restrict__ part_acc, float* __restrict__ part_ml, DecArgs a) {
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int* __restrict__ tickets,
+    DecArgs a) {
   constexpr int KPW = KVF_WAVE / LPK;  // keys per wave per iteration
+  constexpr int UNR = 4;               // iterations whose loads are issued together
   __shared__ float red_acc[WAVES][GC][LPK * 8];
   __shared__ float red_ml[WAVES][GC][2];
+  __shared__ int last_flag;
 
   const int seq = seq_ids ? seq_ids[blockIdx.x] : blockIdx.x;
   if (seq < 0 || seq >= a.n_seqs) return;
@@ -46,6 +50,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
   const int pos = ctx - 1;
   int lo = 0;
   if (a.window > 0 && pos - a.window + 1 > 0) lo = pos - a.window + 1;
+  // the key range [lo, ctx) is cut into `splits` runs of `per` keys, a multiple of the
+  // workgroup's stride; runs past the end are empty and still take part in the merge
   const int nkeys = ctx > lo ? ctx - lo : 0;
   int per = (nkeys + a.splits - 1) / a.splits;
   per = (per + WAVES * KPW - 1) / (WAVES * KPW) * (WAVES * KPW);
@@ -69,39 +75,57 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       load8(q + static_cast<size_t>(tok) * a.q_stride + (kvh * G + g0 + g) * D + e0, qv[g]);
   }
 
-  for (int j = k_begin + wave * KPW + kg; j < k_end; j += WAVES * KPW) {
-    const int blk = j / a.block_size;
-    const int page = blk < a.table_stride ? table[blk] : -1;
-    const bool ok = page >= 0 && page < a.num_blocks;  // uniform over the LPK lanes of a key
-    float kf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    float vf[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (ok && lane_on) {
-      const size_t base =
-          ((static_cast<size_t>(page) * a.KV + kvh) * a.block_size + (j - blk * a.block_size)) * D + e0;
-      load8(k_pages + base, kf);
-      load8(v_pages + base, vf);
+  constexpr int STRIDE = WAVES * KPW;
+  for (int j0 = k_begin + wave * KPW + kg; j0 < k_end; j0 += UNR * STRIDE) {
+    float kf[UNR][8], vf[UNR][8];
+    bool ok[UNR];
+    size_t base[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int j = j0 + u * STRIDE;
+      ok[u] = false;
+      base[u] = 0;
+      if (j < k_end) {
+        const int blk = j / a.block_size;
+        const int page = blk < a.table_stride ? table[blk] : -1;
+        ok[u] = page >= 0 && page < a.num_blocks;
+        base[u] = ((static_cast<size_t>(ok[u] ? page : 0) * a.KV + kvh) * a.block_size +
+                   (j - blk * a.block_size)) * D + e0;
+      }
     }
 #pragma unroll
-    for (int g = 0; g < GC; ++g) {
-      if (g0 + g >= G) break;
-      float s = 0.f;
+    for (int u = 0; u < UNR; ++u) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) s = fmaf(qv[g][e], kf[e], s);
-#pragma unroll
-      for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, KVF_WAVE);
-      if (!ok) continue;
-      s *= a.scale;
-      if (s > m[g]) {
-        const float c = exp_fn<EXACT>(m[g] - s);
-        l[g] *= c;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[g][e] *= c;
-        m[g] = s;
+      for (int e = 0; e < 8; ++e) { kf[u][e] = 0.f; vf[u][e] = 0.f; }
+      if (ok[u] && lane_on) {
+        load8(k_pages + base[u], kf[u]);
+        load8(v_pages + base[u], vf[u]);
       }
-      const float p = exp_fn<EXACT>(s - m[g]);
-      l[g] += p;
+    }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(p, vf[e], acc[g][e]);
+    for (int u = 0; u < UNR; ++u) {
+#pragma unroll
+      for (int g = 0; g < GC; ++g) {
+        if (g0 + g >= G) break;
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s = fmaf(qv[g][e], kf[u][e], s);
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, KVF_WAVE);
+        if (!ok[u]) continue;
+        s *= a.scale;
+        if (s > m[g]) {
+          const float c = exp_fn<EXACT>(m[g] - s);
+          l[g] *= c;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[g][e] *= c;
+          m[g] = s;
+        }
+        const float p = exp_fn<EXACT>(s - m[g]);
+        l[g] += p;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = fmaf(p, vf[u][e], acc[g][e]);
+      }
     }
   }
 
@@ -122,8 +146,6 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       for (int o = LPK; o < KVF_WAVE; o <<= 1) v += __shfl_xor(v, o, KVF_WAVE);
       acc[g][e] = v;
     }
-    m[g] = mm;
-    l[g] = ll;
     if (kg == 0) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) red_acc[wave][g][e0 + e] = acc[g][e];
@@ -156,38 +178,43 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
       if (e == 0) { part_ml[slot * 2] = mm; part_ml[slot * 2 + 1] = ll; }
     }
   }
-}
-
-template <typename T, bool EXACT>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ part_acc,
-                                           const float* __restrict__ part_ml,
-                                           const int* __restrict__ seq_ids,
-                                           const int* __restrict__ cu_q, T* __restrict__ out,
-                                           int H, int D, int splits, int o_stride, int n_seqs) {
-  const int seq = seq_ids ? seq_ids[blockIdx.x] : blockIdx.x;
-  if (seq < 0 || seq >= n_seqs) return;
-  const int head = blockIdx.y;
-  const size_t slot0 = (static_cast<size_t>(blockIdx.x) * H + head) * splits;
-  float mm = -INFINITY;
-  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, part_ml[(slot0 + s) * 2]);
-  const int tok = cu_q[seq];
-  for (int e = threadIdx.x; e < D; e += blockDim.x) {
+  if (a.splits == 1) return;
+  // The workgroup that finishes last for this (sequence, head chunk) merges the splits, in
+  // split order, so the result does not depend on which one that is.  The ticket counts up to
+  // `splits` and is put back to zero by the merging workgroup.
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int t = atomicAdd(tickets + blockIdx.x * gridDim.y + blockIdx.y, 1);
+    last_flag = (t == a.splits - 1);
+  }
+  __syncthreads();
+  if (!last_flag) return;
+  __threadfence();
+  for (int idx = threadIdx.x; idx < GC * LPK * 8; idx += 256) {
+    const int g = idx / (LPK * 8), e = idx - g * (LPK * 8);
+    if (g0 + g >= G || e >= D) continue;
+    const int head = kvh * G + g0 + g;
+    const size_t slot0 = (static_cast<size_t>(blockIdx.x) * a.H + head) * a.splits;
+    float mm = -INFINITY;
+    for (int s = 0; s < a.splits; ++s) mm = fmaxf(mm, __builtin_nontemporal_load(part_ml + (slot0 + s) * 2));
     float ll = 0.f, v = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = part_ml[(slot0 + s) * 2];
+    for (int s = 0; s < a.splits; ++s) {
+      const float ms = __builtin_nontemporal_load(part_ml + (slot0 + s) * 2);
       const float c = (ms == -INFINITY) ? 0.f : exp_fn<EXACT>(ms - mm);
-      ll += part_ml[(slot0 + s) * 2 + 1] * c;
-      v += part_acc[(slot0 + s) * D + e] * c;
+      ll += __builtin_nontemporal_load(part_ml + (slot0 + s) * 2 + 1) * c;
+      v += __builtin_nontemporal_load(part_acc + (slot0 + s) * D + e) * c;
     }
-    Elem<T>::store(out + static_cast<size_t>(tok) * o_stride + head * D + e,
+    Elem<T>::store(out + static_cast<size_t>(tok) * a.o_stride + head * D + e,
                    ll > 0.f ? v / ll : 0.f);
   }
+  if (threadIdx.x == 0) tickets[blockIdx.x * gridDim.y + blockIdx.y] = 0;
 }
 
 template <typename T, bool EXACT>
 int launch(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
            const int* seq_ids, const int* cu_q, const int* ctx_lens, void* out, float* part_acc,
-           float* part_ml, int num_seqs, DecArgs a, hipStream_t s) {
+           float* part_ml, int* tickets, int num_seqs, DecArgs a, hipStream_t s) {
   if (num_seqs <= 0) return 0;
   const int G = a.H / a.KV;
   const int lanes = a.d / 8 + (a.d % 8 ? 1 : 0);
@@ -199,7 +226,7 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
   hipLaunchKernelGGL((attn_decode_kernel<T, LPK, GC, EXACT>), grid, dim3(256), 0, s,              \
                      static_cast<const T*>(q), static_cast<const T*>(k_pages),                    \
                      static_cast<const T*>(v_pages), block_table, seq_ids, cu_q, ctx_lens,        \
-                     static_cast<T*>(out), part_acc, part_ml, a)
+                     static_cast<T*>(out), part_acc, part_ml, tickets, a)
 #define PICK(GC)                                                                                  \
   switch (lpk) {                                                                                  \
     case 2: GO(2, GC); break;                                                                     \
@@ -211,33 +238,30 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
   if (gc == 4) { PICK(4) } else { PICK(8) }
 #undef PICK
 #undef GO
-  int err = kvf_last_error();
-  if (err || a.splits == 1) return err;
-  hipLaunchKernelGGL((attn_decode_combine_kernel<T, EXACT>), dim3(num_seqs, a.H), dim3(64), 0, s,
-                     part_acc, part_ml, seq_ids, cu_q, static_cast<T*>(out), a.H, a.d, a.splits,
-                     a.o_stride, a.n_seqs);
   return kvf_last_error();
 }
 }  // namespace
 
 // dtype: 0 = fp32 (accurate exp), 1 = bf16.  d: multiple of 16, at most 256.
-// With splits > 1, part_acc holds num_seqs*H*splits*d floats and part_ml num_seqs*H*splits*2.
+// With splits > 1, part_acc holds num_seqs*H*splits*d floats, part_ml num_seqs*H*splits*2, and
+// tickets num_seqs * KV * ceil(G / (G <= 4 ? 4 : 8)) ints that are zero before the first call
+// (every call leaves them zero).  Calls that share these buffers must not overlap.
 KVF_EXPORT int kvf_attn_decode(int dtype, const void* q, const void* k_pages, const void* v_pages,
                                const int* block_table, const int* seq_ids, const int* cu_q,
                                const int* ctx_lens, void* out, float* part_acc, float* part_ml,
-                               int num_seqs, int H, int KV, int d, int block_size, int num_blocks,
+                               int* tickets, int num_seqs, int H, int KV, int d, int block_size, int num_blocks,
                                int table_stride, int q_stride, int o_stride, int window,
                                int n_seqs, int splits, float scale, hipStream_t s) {
   if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1)
     return static_cast<int>(hipErrorInvalidValue);
-  if (splits > 1 && (!part_acc || !part_ml)) return static_cast<int>(hipErrorInvalidValue);
+  if (splits > 1 && (!part_acc || !part_ml || !tickets)) return static_cast<int>(hipErrorInvalidValue);
   DecArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
             splits, scale};
   if (dtype == 0)
     return launch<float, true>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
-                               part_acc, part_ml, num_seqs, a, s);
+                               part_acc, part_ml, tickets, num_seqs, a, s);
   if (dtype == 1)
     return launch<bf16_t, false>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
-                                 part_acc, part_ml, num_seqs, a, s);
+                                 part_acc, part_ml, tickets, num_seqs, a, s);
   return static_cast<int>(hipErrorInvalidValue);
 }

@@ -33,7 +33,8 @@ KVF_EXPORT int kvf_embed_bf16(const int* ids, const void* t, float* o, int n, in
 
 // ----------------------------------------------------------------------------- RMS norm
 // y = x * rsqrt(mean(x^2) + eps) * w, all in fp32, rounded once to T on store.
-// x is the fp32 residual stream; `rows` (may be null) gathers input rows; w is fp32 or T.
+// x is the fp32 residual stream; `rows` (may be null) gathers input rows; w is fp32 or T, or
+// null when the weight has been folded into the matrix that consumes y.
 template <typename T, typename W>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
                                const W* __restrict__ w, float eps, T* __restrict__ out, int h,
@@ -54,8 +55,12 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restric
   }
   ss = block_sum(ss, scratch);
   const float r = rsqrtf(ss / static_cast<float>(h) + eps);
-  for (int i = threadIdx.x; i < h; i += blockDim.x)
-    Elem<T>::store(o + i, xr[i] * r * Elem<W>::load(w + i));
+  if (w) {
+    for (int i = threadIdx.x; i < h; i += blockDim.x)
+      Elem<T>::store(o + i, xr[i] * r * Elem<W>::load(w + i));
+  } else {
+    for (int i = threadIdx.x; i < h; i += blockDim.x) Elem<T>::store(o + i, xr[i] * r);
+  }
 }
 
 template <typename T>
@@ -81,40 +86,49 @@ KVF_EXPORT int kvf_rmsnorm_bf16(const float* x, const int* rows, const void* w, 
 }
 
 // ----------------------------------------------------------------------------- SwiGLU gate
-// out[m, i] = silu(gu[m, i]) * gu[m, I + i], silu(x) = x / (1 + exp(-x)), in fp32.
+// out[m, i] = silu(gate) * up with silu(x) = x / (1 + exp(-x)), in fp32.  The input row holds
+// gate and up side by side: gate at 2i and up at 2i + 1 (`paired` != 0, the layout the fused
+// gate/up matrix produces) or gate at i and up at I + i.
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter,
-                                size_t total) {
+                                size_t total, int paired) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t m = idx / inter;
   const int i = static_cast<int>(idx - m * inter);
   const T* row = gu + m * 2 * static_cast<size_t>(inter);
-  const float g = Elem<T>::load(row + i);
-  const float u = Elem<T>::load(row + inter + i);
+  const float g = Elem<T>::load(paired ? row + 2 * i : row + i);
+  const float u = Elem<T>::load(paired ? row + 2 * i + 1 : row + inter + i);
   Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
 }
 template <typename T>
-static int silu_mul_launch(const void* gu, void* out, int m, int inter, hipStream_t s) {
+static int silu_mul_launch(const void* gu, void* out, int m, int inter, int paired,
+                           hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * inter;
   if (total == 0) return 0;
   const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
   hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, s,
-                     static_cast<const T*>(gu), static_cast<T*>(out), inter, total);
+                     static_cast<const T*>(gu), static_cast<T*>(out), inter, total, paired);
   return kvf_last_error();
 }
-KVF_EXPORT int kvf_silu_mul_f32(const void* gu, void* out, int m, int inter, hipStream_t s) {
-  return silu_mul_launch<float>(gu, out, m, inter, s);
+KVF_EXPORT int kvf_silu_mul_f32(const void* gu, void* out, int m, int inter, int paired,
+                                hipStream_t s) {
+  return silu_mul_launch<float>(gu, out, m, inter, paired, s);
 }
-KVF_EXPORT int kvf_silu_mul_bf16(const void* gu, void* out, int m, int inter, hipStream_t s) {
-  return silu_mul_launch<bf16_t>(gu, out, m, inter, s);
+KVF_EXPORT int kvf_silu_mul_bf16(const void* gu, void* out, int m, int inter, int paired,
+                                 hipStream_t s) {
+  return silu_mul_launch<bf16_t>(gu, out, m, inter, paired, s);
 }
 
 // ----------------------------------------------------------------------------- rotary + cache write
 // qkv: [N, (H + 2*KV) * d] rows of q heads, then k heads, then v heads.
-// For token n at position p (cos/sin tables [table_len, rot/2] fp32):
-//   q and k: x'[i] = x[i]*cos[i] - x[i+rot/2]*sin[i];  x'[i+rot/2] = x[i+rot/2]*cos[i] + x[i]*sin[i]
-//   for i < rot/2; elements at or beyond `rot` are copied.  q is rotated in place.
+// A rotary pair is two neighbouring elements (2i, 2i + 1) of a head: the projection matrices
+// are stored with their rows permuted so that what the checkpoint's layout calls elements i and
+// i + rot/2 land there (a dot product of q and k does not care about the order, and v and the
+// output projection are not permuted).  For token n at position p (cos/sin tables
+// [table_len, rot/2] fp32) and i < rot/2:
+//   x'[2i] = x[2i]*cos[i] - x[2i+1]*sin[i];   x'[2i+1] = x[2i+1]*cos[i] + x[2i]*sin[i]
+// elements at or beyond `rot` are copied.  q is rotated in place.
 // Rotated k and v go to the pages: page = block_table[seq_of_token[n], p / block_size];
 // a negative page (padding, or a page already given back) or p outside the table skips the write.
 // Pages are [num_blocks, KV, block_size, d].  With write_kv == 0 only q is rotated.
@@ -151,10 +165,10 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
   for (int t = threadIdx.x; t < q_pairs; t += blockDim.x) {
     const int hh = t / half, i = t - hh * half;
     T* x = row + hh * a.d;
-    const float x1 = Elem<T>::load(x + i), x2 = Elem<T>::load(x + i + half);
+    const float x1 = Elem<T>::load(x + 2 * i), x2 = Elem<T>::load(x + 2 * i + 1);
     const float c = pos_ok ? cs[i] : 1.f, s = pos_ok ? sn[i] : 0.f;
-    Elem<T>::store(x + i, x1 * c - x2 * s);
-    Elem<T>::store(x + i + half, x2 * c + x1 * s);
+    Elem<T>::store(x + 2 * i, x1 * c - x2 * s);
+    Elem<T>::store(x + 2 * i + 1, x2 * c + x1 * s);
   }
   if (page < 0) return;
   // k heads: rotate, write to the page; the unrotated tail is copied
@@ -163,9 +177,9 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
     const int hh = t / half, i = t - hh * half;
     const T* x = row + (a.H + hh) * a.d;
     T* dst = k_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d;
-    const float x1 = Elem<T>::load(x + i), x2 = Elem<T>::load(x + i + half);
-    Elem<T>::store(dst + i, x1 * cs[i] - x2 * sn[i]);
-    Elem<T>::store(dst + i + half, x2 * cs[i] + x1 * sn[i]);
+    const float x1 = Elem<T>::load(x + 2 * i), x2 = Elem<T>::load(x + 2 * i + 1);
+    Elem<T>::store(dst + 2 * i, x1 * cs[i] - x2 * sn[i]);
+    Elem<T>::store(dst + 2 * i + 1, x2 * cs[i] + x1 * sn[i]);
   }
   const int tail = a.d - a.rot;
   for (int t = threadIdx.x; t < a.KV * tail; t += blockDim.x) {

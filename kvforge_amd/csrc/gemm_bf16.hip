@@ -1,17 +1,25 @@
-// C[M, N] = A[M, K] * W[N, K]^T for bf16 operands on the matrix cores (fp32 accumulation),
+// C[M, N] = A[M, K] * W[N, K]^T for bf16 weights on the matrix cores (fp32 accumulation),
 // built for few rows of A: the weight matrix is streamed once per pass of up to 16*MT rows and
 // the kernel is bound by HBM, so all of the chip has to pull on W at once.
 //
 // One workgroup owns 16 rows of W (16 output columns).  Its waves split K: wave w takes the
 // 32-wide k-steps w, w + nw, w + 2nw, ... so neighbouring waves read neighbouring 64-byte pieces
 // of the same rows.  Per k-step a lane loads 16 B of W (row lane%16, k-offset 8*(lane/16)) and
-// 16 B of each 16-row tile of A (row lane%16, same k-offset) and issues one
-// v_mfma_f32_16x16x32_bf16 per tile with W as the first operand, so a lane ends up holding four
-// consecutive output columns of one row of C.  Partial sums of the waves are added in wave order
-// through LDS.  The number of waves depends on N, K and on how many 16-row tiles a pass holds
-// (1, 2, 4 or 8), never on the rows themselves.
+// the matching 8 elements of each 16-row tile of A and issues one v_mfma_f32_16x16x32_bf16 per
+// tile with W as the first operand, so a lane ends up holding four consecutive output columns of
+// one row of C.  Partial sums of the waves are added in wave order through LDS.  The number of
+// waves depends on N, K and on how many 16-row tiles a pass holds, never on the rows themselves.
 //
-// out_kind: 0 store fp32, 1 store bf16, 2 add into fp32 (the residual stream).
+// Left operand (AT): 0 = bf16 activations; 1 = the fp32 residual stream with the RMS norm folded
+// in: y = x * rsqrt(mean(x^2) + eps) is applied as a per-row factor on the accumulators (the
+// norm's weight vector is folded into W's columns when the model is loaded); the sum of squares
+// is taken in fp32 from the same loads that feed the matrix cores.
+//
+// Epilogues (EPI): 0 store fp32; 1 store bf16; 2 add into fp32 (the residual stream);
+// 3 SwiGLU gate: columns come in (gate, up) pairs, out[m, j] = silu(c[2j]) * c[2j+1] as bf16;
+// 4 rotary + cache write for a fused q/k/v projection: neighbouring columns of q and k heads are
+//   rotary pairs; rotated q goes to the output (bf16, q heads only), rotated k and plain v go
+//   straight into the pages of the token's sequence.
 // K must be a multiple of 8 (16-byte loads); a k-step that passes K loads zeros.
 #include "common.h"
 
@@ -19,21 +27,51 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+struct RopeEpi {
+  const int* positions;
+  const int* seq_of_token;
+  const float* cos_t;
+  const float* sin_t;
+  const int* block_table;
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
+};
+
 __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
   uint4 r = make_uint4(0u, 0u, 0u, 0u);
   if (ok) r = *reinterpret_cast<const uint4*>(p);
   return __builtin_bit_cast(bf16x8, r);
 }
 
-// more row tiles per pass mean more registers per lane and more LDS per wave: fewer waves
-constexpr int max_waves(int mt) { return mt <= 2 ? 16 : (mt == 4 ? 8 : 4); }
+// 8 fp32 -> 8 bf16 (round to nearest even); adds their squares to ss
+__device__ __forceinline__ bf16x8 load_frag_f32(const float* p, bool ok, float& ss) {
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (ok) load8(p, v);
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    ss = fmaf(v[2 * i], v[2 * i], ss);
+    ss = fmaf(v[2 * i + 1], v[2 * i + 1], ss);
+    w[i] = static_cast<uint32_t>(f32_to_bf16(v[2 * i])) |
+           (static_cast<uint32_t>(f32_to_bf16(v[2 * i + 1])) << 16);
+  }
+  return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+}
 
-template <int MT, int OUT>
-__global__ __launch_bounds__(max_waves(MT) * KVF_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ A,
-                                                           const bf16_t* __restrict__ W,
-                                                           void* __restrict__ Cv, int M, int N,
-                                                           int K, int lda, int ldc, int m_base) {
-  extern __shared__ float red[];  // [nw][MT][64 lanes][4]
+// more row tiles per pass mean more registers per lane and more LDS per wave: fewer waves; fp32
+// rows take twice the registers while in flight
+constexpr int max_waves(int mt, int at) {
+  return at ? (mt == 1 ? 16 : mt == 2 ? 8 : 4) : (mt <= 2 ? 16 : (mt == 4 ? 8 : 4));
+}
+// k-steps whose loads are in flight together in one wave
+constexpr int depth(int mt, int at) { return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : 4; }
+
+template <int MT, int AT, int EPI>
+__global__ __launch_bounds__(max_waves(MT, AT) * KVF_WAVE) void gemm_skinny_kernel(
+    const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
+    int K, int lda, int ldc, int m_base, float eps, RopeEpi rp) {
+  extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
   const int nw = blockDim.x / KVF_WAVE;
   const int n0 = blockIdx.x * 16;
@@ -41,32 +79,36 @@ __global__ __launch_bounds__(max_waves(MT) * KVF_WAVE) void gemm_skinny_kernel(c
   int wrow = n0 + r16;
   if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
   const bf16_t* wp = W + static_cast<size_t>(wrow) * K + kg * 8;
-  const bf16_t* ap[MT];
+  size_t aoff[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     int arow = m_base + t * 16 + r16;
     if (arow >= M) arow = M - 1;
-    ap[t] = A + static_cast<size_t>(arow) * lda + kg * 8;
+    aoff[t] = static_cast<size_t>(arow) * lda + kg * 8;
   }
+  const bf16_t* Ab = static_cast<const bf16_t*>(Av);
+  const float* Af = static_cast<const float*>(Av);
   f32x4 acc[MT];
+  float ss[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < MT; ++t) { acc[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
 
   const int ksteps = (K + 31) / 32;
   int ks = wave;
-  // four k-steps in flight per wave
-  for (; ks + 3 * nw < ksteps; ks += 4 * nw) {
-    bf16x8 wf[4], af[4][MT];
+  constexpr int U = depth(MT, AT);
+  for (; ks + (U - 1) * nw < ksteps; ks += U * nw) {
+    bf16x8 wf[U], af[U][MT];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < U; ++u) {
       const int k = (ks + u * nw) * 32;
       const bool ok = k + kg * 8 + 8 <= K;
       wf[u] = load_frag(wp + k, ok);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) af[u][t] = load_frag(ap[t] + k, ok);
+      for (int t = 0; t < MT; ++t)
+        af[u][t] = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], af[u][t], acc[t], 0, 0, 0);
@@ -76,13 +118,23 @@ __global__ __launch_bounds__(max_waves(MT) * KVF_WAVE) void gemm_skinny_kernel(c
     const bool ok = k + kg * 8 + 8 <= K;
     const bf16x8 wf = load_frag(wp + k, ok);
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, load_frag(ap[t] + k, ok), acc[t], 0, 0, 0);
+    for (int t = 0; t < MT; ++t) {
+      const bf16x8 af = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc[t], 0, 0, 0);
+    }
   }
-  // lane holds C[row m = r16][cols n0 + 4*kg .. +3] of each tile
+  // lane holds C[row r16][cols n0 + 4*kg .. +3] of each tile
+  float* red_ss = red + nw * MT * KVF_WAVE * 4;
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
+  for (int t = 0; t < MT; ++t) {
     *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * KVF_WAVE + lane) * 4) = acc[t];
+    if (AT) {
+      float v = ss[t];
+      v += __shfl_xor(v, 16, KVF_WAVE);
+      v += __shfl_xor(v, 32, KVF_WAVE);
+      if (kg == 0) red_ss[(wave * MT + t) * 16 + r16] = v;
+    }
+  }
   __syncthreads();
   for (int item = threadIdx.x; item < MT * KVF_WAVE; item += blockDim.x) {
     const int t = item / KVF_WAVE, l = item % KVF_WAVE;
@@ -91,61 +143,157 @@ __global__ __launch_bounds__(max_waves(MT) * KVF_WAVE) void gemm_skinny_kernel(c
       s += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * KVF_WAVE + l) * 4);
     const int m = m_base + t * 16 + l % 16;
     const int n = n0 + 4 * (l / 16);
-    if (m >= M) continue;
+    if (m >= M || n >= N) continue;
+    if (AT) {
+      float tot = 0.f;
+      for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
+      s *= rsqrtf(tot / static_cast<float>(K) + eps);
+    }
+    if (EPI <= 2) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      if (n + r >= N) break;
-      const size_t idx = static_cast<size_t>(m) * ldc + n + r;
-      if (OUT == 0) static_cast<float*>(Cv)[idx] = s[r];
-      if (OUT == 1) static_cast<bf16_t*>(Cv)[idx].bits = f32_to_bf16(s[r]);
-      if (OUT == 2) static_cast<float*>(Cv)[idx] += s[r];
+      for (int r = 0; r < 4; ++r) {
+        if (n + r >= N) break;
+        const size_t idx = static_cast<size_t>(m) * ldc + n + r;
+        if (EPI == 0) static_cast<float*>(Cv)[idx] = s[r];
+        if (EPI == 1) static_cast<bf16_t*>(Cv)[idx].bits = f32_to_bf16(s[r]);
+        if (EPI == 2) static_cast<float*>(Cv)[idx] += s[r];
+      }
+    } else if (EPI == 3) {
+      // N is even and n a multiple of 4: two (gate, up) pairs
+      bf16_t* o = static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n / 2;
+      o[0].bits = f32_to_bf16(s[0] / (1.f + __expf(-s[0])) * s[1]);
+      if (n + 2 < N) o[1].bits = f32_to_bf16(s[2] / (1.f + __expf(-s[2])) * s[3]);
+    } else {
+      // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head
+      const int head = n / rp.d, e = n - head * rp.d;
+      const int p = rp.positions[m];
+      const bool pos_ok = p >= 0 && p < rp.table_len;
+      float o[4] = {s[0], s[1], s[2], s[3]};
+      if (head < rp.H + rp.KV && pos_ok) {
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          const int j = (e + 2 * pr) / 2;
+          if (2 * j + 1 < rp.rot) {
+            const float c = rp.cos_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
+            const float sn = rp.sin_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
+            const float x1 = s[2 * pr], x2 = s[2 * pr + 1];
+            o[2 * pr] = x1 * c - x2 * sn;
+            o[2 * pr + 1] = x2 * c + x1 * sn;
+          }
+        }
+      }
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(f32_to_bf16(o[0])) | (static_cast<uint32_t>(f32_to_bf16(o[1])) << 16);
+      packed.y = static_cast<uint32_t>(f32_to_bf16(o[2])) | (static_cast<uint32_t>(f32_to_bf16(o[3])) << 16);
+      if (head < rp.H) {
+        *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n) = packed;
+      } else if (rp.write_kv && pos_ok) {
+        const int seq = rp.seq_of_token[m];
+        const int blk = p / rp.block_size;
+        int page = -1;
+        if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
+          page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
+        if (page >= 0 && page < rp.num_blocks) {
+          const bool is_k = head < rp.H + rp.KV;
+          const int kvh = is_k ? head - rp.H : head - rp.H - rp.KV;
+          bf16_t* pages = is_k ? rp.k_pages : rp.v_pages;
+          *reinterpret_cast<uint2*>(
+              pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size +
+                       (p - blk * rp.block_size)) * rp.d + e) = packed;
+        }
+      }
     }
   }
 }
 
-template <int MT>
-int launch_mt(const bf16_t* A, const bf16_t* W, void* C, int out_kind, int M, int N, int K,
-              int lda, int ldc, int m_base, int nw, hipStream_t s) {
-  if (nw > max_waves(MT)) nw = max_waves(MT);
-  const dim3 grid((N + 15) / 16), block(nw * KVF_WAVE);
-  const size_t lds = static_cast<size_t>(nw) * MT * KVF_WAVE * 4 * sizeof(float);
-#define GO(OUT)                                                                                    \
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, OUT>), grid, block, lds, s, A, W, C, M, N, K, lda,   \
-                     ldc, m_base)
-  if (out_kind == 0) GO(0);
-  else if (out_kind == 1) GO(1);
-  else GO(2);
-#undef GO
-  return kvf_last_error();
-}
-}  // namespace
+int g_waves_override = 0;
 
 // Waves per workgroup: enough workgroups x waves to keep every CU streaming, at least one
 // k-step per wave, at most 16.
-static int pick_waves(int N, int K) {
+int pick_waves(int N, int K) {
   const int tiles = (N + 15) / 16, ksteps = (K + 31) / 32;
-  int nw = (4096 + tiles - 1) / tiles;
+  int nw = g_waves_override > 0 ? g_waves_override : (4096 + tiles - 1) / tiles;
   if (nw > 16) nw = 16;
   if (nw > ksteps) nw = ksteps;
   if (nw < 1) nw = 1;
   return nw;
 }
 
-KVF_EXPORT int kvf_gemm_bf16(const void* A, const void* W, void* C, int out_kind, int M, int N,
-                             int K, int lda, int ldc, hipStream_t s) {
-  if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || out_kind < 0 || out_kind > 2)
-    return static_cast<int>(hipErrorInvalidValue);
-  const bf16_t* a = static_cast<const bf16_t*>(A);
-  const bf16_t* w = static_cast<const bf16_t*>(W);
+template <int MT, int AT, int EPI>
+int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
+               int m_base, int nw, float eps, const RopeEpi& rp, hipStream_t s) {
+  if (nw > max_waves(MT, AT)) nw = max_waves(MT, AT);
+  const dim3 grid((N + 15) / 16), block(nw * KVF_WAVE);
+  const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
+                     lda, ldc, m_base, eps, rp);
+  return kvf_last_error();
+}
+
+template <int AT, int EPI>
+int launch_rows(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
+                float eps, const RopeEpi& rp, hipStream_t s) {
   const int nw = pick_waves(N, K);
   int err = 0;
   for (int m_base = 0; m_base < M && !err; m_base += 128) {
     const int rows = M - m_base < 128 ? M - m_base : 128;
-    if (rows <= 16) err = launch_mt<1>(a, w, C, out_kind, M, N, K, lda, ldc, m_base, nw, s);
-    else if (rows <= 32) err = launch_mt<2>(a, w, C, out_kind, M, N, K, lda, ldc, m_base, nw, s);
-    else if (rows <= 64) err = launch_mt<4>(a, w, C, out_kind, M, N, K, lda, ldc, m_base, nw, s);
-    else err = launch_mt<8>(a, w, C, out_kind, M, N, K, lda, ldc, m_base, nw, s);
+    if (rows <= 16) err = launch_one<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
+    else if (rows <= 32) err = launch_one<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
+    else if (rows <= 64) err = launch_one<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
+    else err = launch_one<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
   }
   return err;
+}
+
+template <int AT>
+int launch_epi(const void* A, const bf16_t* W, void* C, int epi, int M, int N, int K, int lda,
+               int ldc, float eps, const RopeEpi& rp, hipStream_t s) {
+  switch (epi) {
+    case 0: return launch_rows<AT, 0>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+    case 1: return launch_rows<AT, 1>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+    case 2: return launch_rows<AT, 2>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+    case 3: return launch_rows<AT, 3>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+    case 4: return launch_rows<AT, 4>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+  }
+  return static_cast<int>(hipErrorInvalidValue);
+}
+}  // namespace
+
+// For measurements: force the number of waves per workgroup (0 = choose by shape).
+KVF_EXPORT void kvf_gemm_bf16_set_waves(int waves) { g_waves_override = waves; }
+
+// a_type: 0 = bf16 rows, 1 = fp32 rows normalised by rsqrt(mean(x^2) + eps) in the kernel.
+// epi: 0 store fp32, 1 store bf16, 2 add into fp32, 3 SwiGLU pairs -> bf16 [M, N/2].
+KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, void* C, int epi, int M,
+                             int N, int K, int lda, int ldc, float eps, hipStream_t s) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || epi < 0 || epi > 3 || (epi == 3 && N % 4 != 0))
+    return static_cast<int>(hipErrorInvalidValue);
+  const RopeEpi none{};
+  const bf16_t* w = static_cast<const bf16_t*>(W);
+  if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, none, s);
+  if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, none, s);
+  return static_cast<int>(hipErrorInvalidValue);
+}
+
+// Fused q/k/v projection with rotary and cache write.  W: [(H + 2*KV) * d, K] with q and k rows
+// permuted so that rotary pairs are neighbouring rows.  q_out: [M, ldq >= H * d] bf16.
+KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, void* q_out, int M,
+                                      int K, int lda, int ldq, float eps, const int* positions,
+                                      const int* seq_of_token, const float* cos_t,
+                                      const float* sin_t, const int* block_table, void* k_pages,
+                                      void* v_pages, int H, int KV, int d, int rot, int table_len,
+                                      int block_size, int table_stride, int num_blocks,
+                                      int write_kv, int n_seqs, hipStream_t s) {
+  if (M <= 0) return 0;
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || d % 4 != 0 || rot % 2 != 0 || rot > d || ldq % 4 != 0)
+    return static_cast<int>(hipErrorInvalidValue);
+  const RopeEpi rp{positions, seq_of_token, cos_t, sin_t, block_table,
+                   static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), H, KV, d, rot,
+                   table_len, block_size, table_stride, num_blocks, write_kv, n_seqs};
+  const int N = (H + 2 * KV) * d;
+  const bf16_t* w = static_cast<const bf16_t*>(W);
+  if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, rp, s);
+  if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, rp, s);
+  return static_cast<int>(hipErrorInvalidValue);
 }

@@ -17,6 +17,7 @@ import numpy as np
 import torch
 
 ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup handles
+DECODE_KEYS_PER_SPLIT = 128
 
 
 @dataclass
@@ -64,6 +65,20 @@ class Workspace:
             if self.frozen:
                 raise RuntimeError(f"workspace buffer {name} would grow during graph capture")
             flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = flat
+        return flat[:n].view(shape)
+
+    def zeros(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        """Like ``buf`` for memory whose users leave it zero: cleared once, when it is made."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        flat = self._bufs.get(key)
+        if flat is None or flat.numel() < n:
+            if self.frozen:
+                raise RuntimeError(f"workspace buffer {name} would grow during graph capture")
+            flat = torch.zeros(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = flat
         return flat[:n].view(shape)
 
@@ -128,6 +143,7 @@ class Step:
         self.host_token_ids: np.ndarray | None = None
         self.prefill_seqs: list[int] = []
         self.max_decode_ctx = 0
+        self.max_position = 0
         self._work: dict[int, torch.Tensor | None] = {}
         self._identity_rotary = None
         self.device: torch.device | str = "cuda"
@@ -145,20 +161,30 @@ class Step:
             self._work[group_size] = w
         return w
 
+    def no_rotation(self) -> tuple[torch.Tensor, torch.Tensor]:
+        """cos/sin tables of a rotation by zero, for mixers without rotary positions: one pair
+        per head is "rotated" by the identity."""
+        if self._identity_rotary is None:
+            n = int(self.positions.shape[0]) if self.positions is not None else 1
+            length = max(self.max_position + 1, n, 1)
+            self._identity_rotary = (torch.ones(length, 1, dtype=torch.float32, device=self.device),
+                                     torch.zeros(length, 1, dtype=torch.float32, device=self.device))
+        return self._identity_rotary
+
     def decode_plan(self, H: int, KV: int, d: int, window: int):
         """How many splits of the key range the decode kernel uses, and its workspace."""
         G = H // KV
         chunks = -(-G // (4 if G <= 4 else 8))
-        wgs = max(1, self.n_decode * KV * chunks)
         ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
-        splits = 1
-        if wgs < 256:
-            splits = max(1, min(-(-512 // wgs), ctx // 256, 64))
+        # about DECODE_KEYS_PER_SPLIT keys per workgroup, so that each wave's loads are all in
+        # flight at once; at most 64 splits
+        splits = max(1, min(-(-ctx // DECODE_KEYS_PER_SPLIT), 64))
         if splits == 1:
             return 1, None
         acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)
         ml = self.ws.buf("decode_part_ml", (self.n_decode * H * splits * 2,), torch.float32)
-        return splits, (acc, ml)
+        tickets = self.ws.zeros("decode_tickets", (self.n_decode * KV * chunks,), torch.int32)
+        return splits, (acc, ml, tickets)
 
 
 def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], tables_of, slot_of,
@@ -256,5 +282,6 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
     step.host_token_ids = tok.copy()
     step.prefill_seqs = prefill
     step.max_decode_ctx = int(max((ctx[b] for b in decode), default=0))
+    step.max_position = int(ctx.max()) if Bp else 0
     step._work = {}
     return counts

@@ -87,38 +87,43 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
 
 
 # ------------------------------------------------------------------------------ RMS norm
-def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch.Tensor,
             rows: torch.Tensor | None = None) -> None:
-    """``out[m] = x[rows[m] or m] * rsqrt(mean(x^2) + eps) * weight`` with fp32 math."""
+    """``out[m] = x[rows[m] or m] * rsqrt(mean(x^2) + eps) * weight`` with fp32 math
+    (``weight=None``: no weight, for a norm whose weight is folded into the next matrix)."""
     _check(x, "x", F32, (None, None))
     xr, h = x.shape
     m = out.shape[0]
     _check(out, "out", None, (m, h))
-    _check(weight, "weight", None, (h,))
-    if weight.dtype not in (F32, out.dtype):
-        raise KernelError(f"norm weight must be float32 or {out.dtype}, got {weight.dtype}")
+    if weight is not None:
+        _check(weight, "weight", None, (h,))
+        if weight.dtype not in (F32, out.dtype):
+            raise KernelError(f"norm weight must be float32 or {out.dtype}, got {weight.dtype}")
     if rows is not None:
         _check(rows, "rows", I32, (m,))
     elif m > xr:
         raise KernelError("rmsnorm: more output rows than input rows")
     f = _fn("elementwise", f"kvf_rmsnorm_{_suffix(out.dtype)}",
             [c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p])
-    _ok(f(x.data_ptr(), rows.data_ptr() if rows is not None else None, weight.data_ptr(),
-          1 if weight.dtype == F32 else 0, float(eps), out.data_ptr(), m, h, xr, _stream()),
-        "rmsnorm")
+    _ok(f(x.data_ptr(), rows.data_ptr() if rows is not None else None,
+          weight.data_ptr() if weight is not None else None,
+          1 if weight is not None and weight.dtype == F32 else 0, float(eps), out.data_ptr(),
+          m, h, xr, _stream()), "rmsnorm")
 
 
 # ------------------------------------------------------------------------------ SwiGLU gate
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """``out = silu(gate_up[:, :I]) * gate_up[:, I:]``."""
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, paired: bool = False) -> None:
+    """``out[:, i] = silu(gate_i) * up_i`` where the input row holds gate at ``i`` and up at
+    ``I + i``, or, with ``paired``, gate at ``2i`` and up at ``2i + 1``."""
     m, two_i = gate_up.shape
     if two_i % 2:
         raise KernelError("silu_mul: input width must be even")
     _check(gate_up, "gate_up", None, (m, two_i))
     _check(out, "out", gate_up.dtype, (m, two_i // 2))
     f = _fn("elementwise", f"kvf_silu_mul_{_suffix(out.dtype)}",
-            [c_void_p, c_void_p, c_int, c_int, c_void_p])
-    _ok(f(gate_up.data_ptr(), out.data_ptr(), m, two_i // 2, _stream()), "silu_mul")
+            [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p])
+    _ok(f(gate_up.data_ptr(), out.data_ptr(), m, two_i // 2, 1 if paired else 0, _stream()),
+        "silu_mul")
 
 
 # ------------------------------------------------------------------------------ rotary + cache
@@ -127,7 +132,8 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
                  k_pages: torch.Tensor, v_pages: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, write_kv: bool = True) -> None:
     """Rotate q (in place) and k by the cos/sin rows of each token's position; write rotated k
-    and v into the pages named by the token's sequence row of ``block_table``."""
+    and v into the pages named by the token's sequence row of ``block_table``.  Rotary pairs
+    are neighbouring elements ``(2i, 2i + 1)`` of a head."""
     n = qkv.shape[0]
     H, KV, d = num_heads, num_kv_heads, head_dim
     _check(qkv, "qkv", None, (n, (H + 2 * KV) * d))
@@ -155,10 +161,36 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 
 
 # ------------------------------------------------------------------------------ matrix products
-_OUT_KIND = {"f32": 0, "bf16": 1, "add": 2}
-
 # Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.
 SKINNY_MAX_M = 128
+_GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
+
+
+def _gemm_operands(a, w, out, n_out):
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+        raise KernelError("gemm takes 2-D tensors")
+    m, k = a.shape
+    n, k2 = w.shape
+    if k != k2 or tuple(out.shape) != (m, n_out(n)):
+        raise KernelError(f"gemm shapes do not agree: a {list(a.shape)}, w {list(w.shape)}, "
+                          f"out {list(out.shape)}")
+    _check(a, "a", None, None, contiguous=False)
+    _check(w, "w")
+    _check(out, "out", None, None, contiguous=False)
+    if a.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: rows of a and out must be dense")
+    lda = a.stride(0) if m > 1 else k
+    ldc = out.stride(0) if m > 1 else out.shape[1]
+    return m, n, k, lda, ldc
+
+
+def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False) -> bool:
+    """Whether the MFMA weight-streaming kernel takes these operands: bf16 weights, bf16 rows
+    (or, with ``rms``, fp32 rows), 16-byte aligned rows, at most ``SKINNY_MAX_M`` of them."""
+    m, k = a.shape
+    lda = a.stride(0) if m > 1 else k
+    return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and k % 8 == 0 and lda % 8 == 0
+            and m <= SKINNY_MAX_M)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -167,31 +199,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     ``a: [M, K]`` (row stride may exceed K), ``w: [N, K]`` contiguous, ``out: [M, N]``.
     bf16 x bf16 runs on MFMA with fp32 accumulation; any operand in fp32 runs the fp32
     vector-ALU kernel (true 32-bit multiply and accumulate)."""
-    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
-        raise KernelError("gemm takes 2-D tensors")
-    m, k = a.shape
-    n, k2 = w.shape
-    if k != k2 or tuple(out.shape) != (m, n):
-        raise KernelError(f"gemm shapes do not agree: a {list(a.shape)}, w {list(w.shape)}, "
-                          f"out {list(out.shape)}")
-    _check(a, "a", None, None, contiguous=False)
-    _check(w, "w")
-    _check(out, "out", None, None, contiguous=False)
-    if a.stride(1) != 1 or out.stride(1) != 1:
-        raise KernelError("gemm: rows of a and out must be dense")
+    m, n, k, lda, ldc = _gemm_operands(a, w, out, lambda n: n)
     if accumulate and out.dtype != F32:
         raise KernelError("gemm: accumulation needs an fp32 output")
     if m == 0:
         return
-    lda, ldc = a.stride(0) if m > 1 else k, out.stride(0) if m > 1 else n
     out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)
     if not accumulate:
         _tcode(out.dtype)
-    if a.dtype == BF16 and w.dtype == BF16 and _bf16_gemm_ok(k, lda):
+    if a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0:
         if m <= SKINNY_MAX_M or out_kind == 0:
-            f = _fn("gemm_bf16", "kvf_gemm_bf16",
-                    [c_void_p, c_void_p, c_void_p] + [c_int] * 6 + [c_void_p])
-            _ok(f(a.data_ptr(), w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc,
+            f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
+            _ok(f(a.data_ptr(), 0, w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
                   _stream()), "gemm_bf16")
         elif accumulate:
             # many rows: the library's bf16 product (as the reference's engine uses one), then
@@ -206,9 +225,84 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
           m, n, k, lda, ldc, _stream()), "gemm_generic")
 
 
-def _bf16_gemm_ok(k: int, lda: int) -> bool:
-    """The MFMA kernel loads 16 bytes at a time: K and the row stride in steps of 8."""
-    return k % 8 == 0 and lda % 8 == 0
+def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: float | None = None,
+               silu_pairs: bool = False, accumulate: bool = False) -> None:
+    """The MFMA weight-streaming product with work folded in at both ends.
+
+    ``rms_eps``: ``a`` is the fp32 residual stream and each row is scaled by
+    ``rsqrt(mean(a^2) + eps)`` (the norm's weight is already folded into ``w``).
+    ``silu_pairs``: columns are (gate, up) pairs and ``out[:, j] = silu(c[2j]) * c[2j+1]``,
+    ``out: [M, N/2]`` bf16.  Callers check ``bf16_kernel_takes`` first."""
+    rms = rms_eps is not None
+    m, n, k, lda, ldc = _gemm_operands(a, w, out, (lambda n: n // 2) if silu_pairs else (lambda n: n))
+    if not bf16_kernel_takes(a, w, rms):
+        raise KernelError("gemm_fused: operands do not fit the MFMA kernel")
+    if silu_pairs:
+        if n % 4 or out.dtype != BF16 or accumulate:
+            raise KernelError("gemm_fused: SwiGLU pairs need N in steps of 4 and a bf16 output")
+        epi = 3
+    elif accumulate:
+        if out.dtype != F32:
+            raise KernelError("gemm_fused: accumulation needs an fp32 output")
+        epi = 2
+    else:
+        epi = 0 if out.dtype == F32 else 1
+        _tcode(out.dtype)
+    if m == 0:
+        return
+    f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
+    _ok(f(a.data_ptr(), 1 if rms else 0, w.data_ptr(), out.data_ptr(), epi, m, n, k, lda, ldc,
+          float(rms_eps or 0.0), _stream()), "gemm_bf16")
+
+
+def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
+                  seq_of_token: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                  block_table: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                  num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True,
+                  rms_eps: float | None = None) -> None:
+    """Fused q/k/v projection: ``a @ w.T`` with rotary applied to q and k (neighbouring columns
+    are pairs), rotated q stored to ``q_out [M, H*d]`` and rotated k and v written into the
+    pages.  ``rms_eps`` as in ``gemm_fused``."""
+    H, KV, d = num_heads, num_kv_heads, head_dim
+    rms = rms_eps is not None
+    m, k = a.shape
+    _check(a, "a", None, (m, k), contiguous=False)
+    _check(w, "w", BF16, ((H + 2 * KV) * d, k))
+    if not bf16_kernel_takes(a, w, rms) or a.stride(1) != 1:
+        raise KernelError("gemm_qkv_rope: operands do not fit the MFMA kernel")
+    _check(q_out, "q_out", BF16, (m, H * d))
+    _check(positions, "positions", I32, (None,))
+    _check(seq_of_token, "seq_of_token", I32, (None,))
+    if positions.shape[0] < m or seq_of_token.shape[0] < m:
+        raise KernelError("gemm_qkv_rope: positions / seq_of_token shorter than the batch")
+    _check(cos, "cos", F32, (None, None))
+    _check(sin, "sin", F32, tuple(cos.shape))
+    table_len, half = cos.shape
+    if 2 * half > d or d % 4:
+        raise KernelError(f"gemm_qkv_rope: rotary width {2 * half} / head_dim {d} not supported")
+    _check(block_table, "block_table", I32, (None, None))
+    _check(k_pages, "k_pages", BF16, (None, KV, None, d))
+    _check(v_pages, "v_pages", BF16, tuple(k_pages.shape))
+    nb, _, bs, _ = k_pages.shape
+    if m == 0:
+        return
+    f = _fn("gemm_bf16", "kvf_gemm_bf16_qkv_rope",
+            [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float]
+            + [c_void_p] * 7 + [c_int] * 10 + [c_void_p])
+    _ok(f(a.data_ptr(), 1 if rms else 0, w.data_ptr(), q_out.data_ptr(), m, k,
+          a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d, float(rms_eps or 0.0),
+          positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+          block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, 2 * half,
+          table_len, bs, block_table.shape[1], nb, 1 if write_kv else 0, block_table.shape[0],
+          _stream()), "gemm_qkv_rope")
+
+
+def set_gemm_waves(waves: int) -> None:
+    """Measurement aid: force the waves per workgroup of the MFMA kernel (0 = by shape)."""
+    lib = library.load("gemm_bf16")
+    lib.kvf_gemm_bf16_set_waves.argtypes = [c_int]
+    lib.kvf_gemm_bf16_set_waves.restype = None
+    lib.kvf_gemm_bf16_set_waves(int(waves))
 
 
 # ------------------------------------------------------------------------------ attention
@@ -267,23 +361,27 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
             raise KernelError("attn_decode: seq_ids shorter than num_seqs")
     elif num_seqs > n_seqs:
         raise KernelError("attn_decode: more sequences than block-table rows")
-    pa = pm = None
+    pa = pm = tk = None
     if splits > 1:
         if workspace is None:
             raise KernelError("attn_decode: splits > 1 need a workspace")
-        pa, pm = workspace
+        pa, pm, tk = workspace
         _check(pa, "workspace[0]", F32)
         _check(pm, "workspace[1]", F32)
-        if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
+        _check(tk, "workspace[2]", I32)
+        G = H // KV
+        chunks = -(-G // (4 if G <= 4 else 8))
+        if (pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2
+                or tk.numel() < num_seqs * KV * chunks):
             raise KernelError("attn_decode: workspace too small")
     nb, _, bs, _ = k_pages.shape
     f = _fn("attn_decode", "kvf_attn_decode",
-            [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+            [c_int] + [c_void_p] * 11 + [c_int] * 12 + [c_float, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
           cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
           pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
-          num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
+          tk.data_ptr() if tk is not None else None, num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
           int(window), n_seqs, int(splits), float(scale), _stream()), "attn_decode")
 
 

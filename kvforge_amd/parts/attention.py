@@ -52,9 +52,33 @@ class PagedAttention(Mixer):
         q, k, v = (tensors[self._name(f"{n}_proj.weight")] for n in "qkv")
         if not (q.dtype == k.dtype == v.dtype):
             q, k, v = q.float(), k.float(), v.float()
+        # The kernels rotate neighbouring elements (2i, 2i+1); the checkpoint pairs element i
+        # with i + rot/2.  Permuting the rows of the q and k projections inside each head moves
+        # the checkpoint's pairs next to each other; q.k does not depend on the order, v and the
+        # output projection keep theirs.
+        perm = self.pair_permutation()
+        q = q.view(self.H, self.d, -1)[:, perm].reshape(self.H * self.d, -1)
+        k = k.view(self.KV, self.d, -1)[:, perm].reshape(self.KV * self.d, -1)
         # one product for the three projections: rows of q heads, then k heads, then v heads
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
         self.w_o = tensors[self._name("o_proj.weight")]
+        self.norm_eps = None
+
+    def pair_permutation(self) -> torch.Tensor:
+        """``perm[new] = old`` within a head: new elements 2i and 2i+1 are the checkpoint's
+        elements i and i + rot/2; elements beyond the rotary width stay."""
+        rot = self.rotary.rot_dim if self.rotary is not None else 0
+        perm = torch.arange(self.d)
+        for i in range(rot // 2):
+            perm[2 * i], perm[2 * i + 1] = i, i + rot // 2
+        return perm
+
+    def absorb_norm(self, norm) -> bool:
+        if self.norm_eps is not None or not getattr(norm, "foldable_into", lambda m: False)(self.w_qkv):
+            return False
+        self.w_qkv = (self.w_qkv.float() * norm.weight.float()[None, :]).to(torch.bfloat16).contiguous()
+        self.norm_eps = norm.eps
+        return True
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         mods = {"elementwise", "gemm_generic", "attn_generic", "attn_decode"}
@@ -66,21 +90,30 @@ class PagedAttention(Mixer):
         return sum(t.numel() * t.element_size() for t in (self.w_qkv, self.w_o) if t is not None)
 
     def forward(self, x, step, layer: LayerState, residual) -> None:
+        """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""
         n = x.shape[0]
         H, KV, d = self.H, self.KV, self.d
         ws = step.ws
-        qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), x.dtype)
-        ops.gemm(x, self.w_qkv, qkv)
+        act = step.act_dtype
         table = step.block_tables[layer.group]
-        if self.rotary is not None:
-            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, self.rotary.cos,
-                             self.rotary.sin, table, layer.k_pages, layer.v_pages, H, KV, d,
-                             write_kv=layer.owns_cache)
+        cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else step.no_rotation()
+        rms = self.norm_eps
+        if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None) and layer.k_pages.dtype == torch.bfloat16:
+            # one kernel: (norm,) projection, rotary, cache write
+            qkv = ws.buf("q_rot", (n, H * d), act)
+            ops.gemm_qkv_rope(x, self.w_qkv, qkv, step.positions, step.seq_of_token, cos, sin, table,
+                              layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache,
+                              rms_eps=rms)
         else:
-            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, step.unit_cos(),
-                             step.zero_sin(), table, layer.k_pages, layer.v_pages, H, KV, d,
-                             write_kv=layer.owns_cache)
-        out = ws.buf("attn_out", (n, H * d), x.dtype)
+            if rms is not None:
+                normed = ws.buf("normed", (n, self.hidden), act)
+                ops.rmsnorm(x, None, rms, normed)
+                x = normed
+            qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), act)
+            ops.gemm(x, self.w_qkv, qkv)
+            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
+                             layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache)
+        out = ws.buf("attn_out", (n, H * d), act)
         window = self.window or 0
         work = step.prefill_work(H // KV)
         if work is not None:

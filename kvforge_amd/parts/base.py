@@ -82,6 +82,12 @@ class Part:
         """Bytes of weights this part reads in one step."""
         return 0
 
+    def absorb_norm(self, norm: "Norm") -> bool:
+        """Offer the norm that feeds this part.  A part that can apply it inside its own first
+        kernel takes what it needs from ``norm`` and returns True; from then on its ``forward``
+        is handed the fp32 residual stream instead of normalised activations."""
+        return False
+
     def _name(self, local: str) -> str:
         return f"{self.prefix}.{local}" if self.prefix else local
 

@@ -13,12 +13,27 @@ class PreNormBlock(Block):
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward) -> None:
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 
+        self.mixer_takes_residual = self.ffn_takes_residual = False
+
     def parts(self) -> list[Part]:
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
+    def load(self, tensors) -> None:
+        super().load(tensors)
+        # a part may apply the norm in front of it inside its own first kernel
+        self.mixer_takes_residual = self.mixer.absorb_norm(self.mixer_norm)
+        self.ffn_takes_residual = self.ffn.absorb_norm(self.ffn_norm)
+
     def forward(self, residual, step, layer: LayerState) -> None:
-        x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
-        self.mixer_norm.forward(residual, x)
-        self.mixer.forward(x, step, layer, residual)
-        self.ffn_norm.forward(residual, x)
-        self.ffn.forward(x, step, residual)
+        if self.mixer_takes_residual:
+            self.mixer.forward(residual, step, layer, residual)
+        else:
+            x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
+            self.mixer_norm.forward(residual, x)
+            self.mixer.forward(x, step, layer, residual)
+        if self.ffn_takes_residual:
+            self.ffn.forward(residual, step, residual)
+        else:
+            x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
+            self.ffn_norm.forward(residual, x)
+            self.ffn.forward(x, step, residual)

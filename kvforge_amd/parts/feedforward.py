@@ -27,9 +27,19 @@ class SwiGLU(FeedForward):
         g, u = tensors[self._name("gate_proj.weight")], tensors[self._name("up_proj.weight")]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        # one product for gate and up: rows [0, I) are gate, rows [I, 2I) are up
-        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        # one product for gate and up, rows interleaved: row 2i is gate_i, row 2i+1 is up_i, so
+        # a kernel that holds neighbouring output columns holds a whole (gate, up) pair
+        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
         self.w_down = tensors[self._name("down_proj.weight")]
+        self.norm_eps = None
+
+    def absorb_norm(self, norm) -> bool:
+        if self.norm_eps is not None or not getattr(norm, "foldable_into", lambda m: False)(self.w_gate_up):
+            return False
+        self.w_gate_up = (self.w_gate_up.float() * norm.weight.float()[None, :]).to(
+            torch.bfloat16).contiguous()
+        self.norm_eps = norm.eps
+        return True
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         mods = {"elementwise", "gemm_generic"}
@@ -42,9 +52,19 @@ class SwiGLU(FeedForward):
                    if t is not None)
 
     def forward(self, x, step, residual) -> None:
+        """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""
         n = x.shape[0]
-        gu = step.ws.buf("gate_up", (n, 2 * self.inter), x.dtype)
-        ops.gemm(x, self.w_gate_up, gu)
-        act = step.ws.buf("ffn_act", (n, self.inter), x.dtype)
-        ops.silu_mul(gu, act)
+        ws, dt, rms = step.ws, step.act_dtype, self.norm_eps
+        act = ws.buf("ffn_act", (n, self.inter), dt)
+        if ops.bf16_kernel_takes(x, self.w_gate_up, rms is not None) and self.inter % 2 == 0:
+            # one kernel: (norm,) gate/up projection, SwiGLU gate
+            ops.gemm_fused(x, self.w_gate_up, act, rms_eps=rms, silu_pairs=True)
+        else:
+            if rms is not None:
+                normed = ws.buf("normed", (n, self.hidden), dt)
+                ops.rmsnorm(x, None, rms, normed)
+                x = normed
+            gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
+            ops.gemm(x, self.w_gate_up, gu)
+            ops.silu_mul(gu, act, paired=True)
         ops.gemm(act, self.w_down, residual, accumulate=True)

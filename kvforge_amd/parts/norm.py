@@ -31,3 +31,9 @@ class RMSNorm(Norm):
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
         ops.rmsnorm(x, self.weight, self.eps, out, rows)
+
+    def foldable_into(self, matrix: torch.Tensor) -> bool:
+        """Whether this norm's weight may be multiplied into the columns of a bf16 matrix: only
+        when it is itself held in bf16 (a weight stored in 32-bit stays a 32-bit multiply)."""
+        return (self.weight is not None and self.weight.dtype == torch.bfloat16
+                and matrix.dtype == torch.bfloat16 and matrix.shape[1] == self.width)

@@ -69,6 +69,9 @@ def test_silu_mul(dtype):
     ops().silu_mul(gu.to(DEV), out)
     want = torch.nn.functional.silu(gu[:, :176].float()) * gu[:, 176:].float()
     torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    ops().silu_mul(gu.to(DEV), out, paired=True)       # gate at 2i, up at 2i + 1
+    want = torch.nn.functional.silu(gu[:, 0::2].float()) * gu[:, 1::2].float()
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
 
 
 @pytest.mark.parametrize("ta", DTYPES)
@@ -124,6 +127,96 @@ def test_gemm_bf16_mfma(m, n, k):
     out2 = torch.empty(m, n, device=DEV)
     ops().gemm(wide.to(DEV)[:, 8:k + 8], w.to(DEV), out2)
     torch.testing.assert_close(out2.double().cpu(), want, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("m", [1, 8, 20, 64, 128])
+@pytest.mark.parametrize("n,k", [(352, 96), (512, 2048), (48, 40)])
+def test_gemm_fused_norm_and_gate(m, n, k):
+    """The MFMA kernel with the RMS norm folded into its left operand (fp32 rows, factor
+    rsqrt(mean(x^2) + eps) per row) and with the SwiGLU gate folded into its store."""
+    g = torch.Generator().manual_seed(m * 7 + n + k)
+    x = torch.randn(m, k, generator=g) * 3
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    eps = 1e-5
+    xn = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    want = xn.double() @ w.double().T
+    out = torch.empty(m, n, device=DEV)
+    ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
+    torch.testing.assert_close(out.double().cpu(), want, atol=2e-2, rtol=2e-2)   # rows are rounded to bf16
+    res = torch.randn(m, n, generator=g)
+    acc = res.clone().to(DEV)
+    ops().gemm_fused(x.to(DEV), w.to(DEV), acc, rms_eps=eps, accumulate=True)
+    torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=2e-2, rtol=2e-2)
+    gate = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_fused(x.to(DEV), w.to(DEV), gate, rms_eps=eps, silu_pairs=True)
+    want_gate = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+    torch.testing.assert_close(gate.double().cpu(), want_gate, atol=2e-2, rtol=3e-2)
+    xb = xn.to(torch.bfloat16)
+    ops().gemm_fused(xb.to(DEV), w.to(DEV), gate, silu_pairs=True)
+    wantb = xb.double() @ w.double().T
+    torch.testing.assert_close(gate.double().cpu(), torch.nn.functional.silu(wantb[:, 0::2]) * wantb[:, 1::2],
+                               atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("m", [1, 9, 40])
+@pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16),
+                                            (32, 8, 64, 64, 16)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
+    """The fused projection + rotary + cache write against projection (MFMA kernel), then the
+    rotary/cache-write kernel: same q, same pages."""
+    k = 96
+    g = torch.Generator().manual_seed(m + d)
+    x = torch.randn(m, k, generator=g)
+    w = (torch.randn((H + 2 * KV) * d, k, generator=g) / 6).to(torch.bfloat16).to(DEV)
+    positions = torch.randint(0, min(60, 12 * bs), (m,), generator=g, dtype=torch.int32)
+    positions[0] = 5
+    seq_of = torch.randint(0, 3, (m,), generator=g, dtype=torch.int32)
+    seq_of[0] = 0
+    nb = 40
+    table = torch.randperm(nb, generator=g)[:3 * 10].reshape(3, 10).to(torch.int32)
+    table[1, 2] = -1                                   # a page that was given back
+    inv_freq = plain.rope_inv_freq(rot, 10000.0)
+    cos_full, sin_full = plain.rope_cos_sin(torch.arange(64), inv_freq)
+    cos_t, sin_t = cos_full[:, : rot // 2].contiguous().to(DEV), sin_full[:, : rot // 2].contiguous().to(DEV)
+    eps = 1e-5
+    if rms:
+        a = x.to(DEV)
+        normed = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
+        ops().rmsnorm(a, None, eps, normed)
+        ref_in = normed
+    else:
+        a = x.to(torch.bfloat16).to(DEV)
+        ref_in = a
+    qkv = torch.empty(m, (H + 2 * KV) * d, dtype=torch.bfloat16, device=DEV)
+    ops().gemm(ref_in, w, qkv)
+    kp_ref = torch.zeros(nb, KV, bs, d, dtype=torch.bfloat16, device=DEV)
+    vp_ref = torch.zeros_like(kp_ref)
+    ops().rope_kvwrite(qkv, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV), kp_ref,
+                       vp_ref, H, KV, d)
+    kp, vp = torch.zeros_like(kp_ref), torch.zeros_like(kp_ref)
+    q = torch.empty(m, H * d, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_qkv_rope(a, w, q, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV), kp,
+                        vp, H, KV, d, rms_eps=eps if rms else None)
+    # the fused kernel rotates fp32 accumulators, the reference rounds the projection to bf16
+    # first; with fp32 rows the rounding of the normalised input differs as well
+    t = dict(atol=3e-2, rtol=3e-2)
+    torch.testing.assert_close(q.float().cpu(), qkv[:, :H * d].float().cpu(), **t)
+    # two tokens of one sequence at one position write the same slot: compare slots hit once
+    slots = {}
+    for i in range(m):
+        slots.setdefault((int(seq_of[i]), int(positions[i])), []).append(i)
+    once = torch.zeros(nb, bs, dtype=torch.bool)
+    for (sq, pos), toks in slots.items():
+        page = int(table[sq, pos // bs]) if pos // bs < table.shape[1] else -1   # beyond the table: skipped
+        if len(toks) == 1 and page >= 0:
+            once[page, pos % bs] = True
+    sel = once[:, None, :, None].expand(nb, KV, bs, d)
+    torch.testing.assert_close(kp.float().cpu()[sel], kp_ref.float().cpu()[sel], **t)
+    torch.testing.assert_close(vp.float().cpu()[sel], vp_ref.float().cpu()[sel], **t)
+    assert once.any()
+    untouched = (kp_ref.float().cpu().abs().sum((1, 3)) == 0)
+    assert (kp.float().cpu().abs().sum((1, 3))[untouched] == 0).all()
 
 
 def test_gemm_bf16_rows_do_not_depend_on_neighbours():
@@ -231,7 +324,7 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
 @pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
                                         (4, 4, 80, 16), (32, 8, 64, 16), (8, 2, 128, 16),
                                         (12, 1, 112, 16), (2, 1, 256, 32)])
-@pytest.mark.parametrize("splits", [1, 3])
+@pytest.mark.parametrize("splits", [1, 3, 7])
 @pytest.mark.parametrize("window", [0, 11])
 def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     seq_lens = [7, 13, 1, 20, 300, 64]  # tests/test_paged_attention.py:61 of the reference + long
@@ -245,7 +338,8 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     ctx = torch.tensor(seq_lens, dtype=torch.int32)
     scale = 1 / math.sqrt(d)
     want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
-    ws = (torch.empty(n * H * splits * d, device=DEV), torch.empty(n * H * splits * 2, device=DEV))
+    ws = (torch.empty(n * H * splits * d, device=DEV), torch.empty(n * H * splits * 2, device=DEV),
+          torch.zeros(n * H, dtype=torch.int32, device=DEV))
     out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
     ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, n,
                       cu.to(DEV), ctx.to(DEV), out, H, KV, d, scale, window, splits, ws)
@@ -259,6 +353,7 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     got = out2.float().cpu()
     torch.testing.assert_close(got[[4, 1]], want[[4, 1]], **tol(dtype))
     assert (got[[0, 2, 3, 5]] == 5.0).all()
+    assert int(ws[2].abs().sum()) == 0          # the tickets are left at zero
 
 
 def test_attn_far_key_stands_out():
@@ -282,7 +377,8 @@ def test_attn_far_key_stands_out():
         # the far key's value dominates
         assert (want.reshape(H, d)[0] - paged.values[0][far, 0]).abs().max() < 0.05
         for splits in (1, 4):
-            ws = (torch.empty(H * splits * d, device=DEV), torch.empty(H * splits * 2, device=DEV))
+            ws = (torch.empty(H * splits * d, device=DEV), torch.empty(H * splits * 2, device=DEV),
+                  torch.zeros(H, dtype=torch.int32, device=DEV))
             out = torch.zeros(1, H * d, device=DEV)
             ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
                               None, 1, cu.to(DEV), ctx.to(DEV), out, H, KV, d, 1 / math.sqrt(d), 0,
@@ -321,9 +417,17 @@ def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
     kf = qkv[:, H * d:(H + KV) * d].float().reshape(n, KV, d)
     vf = qkv[:, (H + KV) * d:].float().reshape(n, KV, d)
 
+    # the kernel pairs neighbouring elements: element 2i / 2i+1 of its layout is what the plain
+    # half-split formula calls element i / i + rot/2
+    perm = torch.arange(d)
+    for i in range(rot // 2):
+        perm[2 * i], perm[2 * i + 1] = i, i + rot // 2
+    inv = torch.argsort(perm)
+
     def rot_part(x):
-        r = plain.apply_rope(x[..., :rot], cos, sin)
-        return torch.cat([r, x[..., rot:]], -1)
+        half_split = x[..., inv]
+        r = plain.apply_rope(half_split[..., :rot], cos, sin)
+        return torch.cat([r, half_split[..., rot:]], -1)[..., perm]
 
     want_q, want_k = rot_part(qf), rot_part(kf)
     got_q = dev_qkv[:, :H * d].float().cpu().reshape(n, H, d)

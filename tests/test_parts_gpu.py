@@ -80,7 +80,7 @@ def test_swiglu_part(dtype):
     x = rand(9, 48, seed=6).to(dtype)
     res = rand(9, 48, seed=7)
     step = Step()
-    step.ws = Workspace(DEV)
+    step.ws, step.act_dtype = Workspace(DEV), dtype
     residual = res.clone().to(DEV)
     part.forward(x.to(DEV), step, residual)
     want = res + plain.swiglu(x.float(), *(w[f"m.{n}_proj.weight"] for n in ("gate", "up", "down")))

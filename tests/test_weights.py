@@ -51,13 +51,25 @@ def test_loading_keeps_stored_precision(tmp_path):
     assert runtime_dtype(torch.int64, torch.bfloat16) == torch.int32
     assert runtime_dtype(torch.float16, torch.bfloat16) == torch.bfloat16
     assert runtime_dtype(torch.float16, torch.float32) == torch.float32
-    # fused projections keep the order q, k, v and gate, up
+    # fused projections: q, k, v stacked with rotary pairs made neighbours inside each q and k
+    # head; gate and up interleaved row by row
     blk = m32.spec.blocks[1]
     p = "model.layers.1."
-    assert torch.equal(blk.mixer.w_qkv, torch.cat([w[p + f"self_attn.{n}_proj.weight"].float()
-                                                   for n in "qkv"]))
-    assert torch.equal(blk.ffn.w_gate_up, torch.cat([w[p + "mlp.gate_proj.weight"].float(),
-                                                     w[p + "mlp.up_proj.weight"].float()]))
+    perm = blk.mixer.pair_permutation()
+    assert perm.tolist() == [0, 8, 1, 9, 2, 10, 3, 11, 4, 12, 5, 13, 6, 14, 7, 15]
+    q = w[p + "self_attn.q_proj.weight"].float().view(4, 16, 64)[:, perm].reshape(64, 64)
+    k = w[p + "self_attn.k_proj.weight"].float().view(2, 16, 64)[:, perm].reshape(32, 64)
+    assert torch.equal(blk.mixer.w_qkv, torch.cat([q, k, w[p + "self_attn.v_proj.weight"].float()]))
+    assert torch.equal(blk.ffn.w_gate_up[0::2], w[p + "mlp.gate_proj.weight"].float())
+    assert torch.equal(blk.ffn.w_gate_up[1::2], w[p + "mlp.up_proj.weight"].float())
+    # under bf16 the norm in front of a projection is folded into its columns; fp32 keeps it apart
+    blk16 = m.spec.blocks[1]
+    assert blk16.mixer_takes_residual and blk16.ffn_takes_residual and blk16.mixer.norm_eps == 1e-5
+    gamma = w[p + "post_attention_layernorm.weight"].float()
+    want = (torch.stack([w[p + "mlp.gate_proj.weight"].float(), w[p + "mlp.up_proj.weight"].float()], 1)
+            .reshape(352, 64) * gamma[None]).to(torch.bfloat16)
+    assert torch.equal(blk16.ffn.w_gate_up, want)
+    assert not blk.mixer_takes_residual and not m32.spec.blocks[0].ffn_takes_residual
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
