@@ -86,7 +86,12 @@ class CacheManager:
         self.pools = [BlockPool(n) for n in counts]
         self.watermark_blocks = [int(watermark * n) for n in counts]
         self._tables: list[dict[str, list[int]]] = [{} for _ in self.groups]
+        # per group and request: pages [0, n) of the table have been given back (windows only)
+        self._released: list[dict[str, int]] = [{} for _ in self.groups]
         self._num_tokens: dict[str, int] = {}
+        # a number per allocation, so that a request id used again is told from its former self
+        self._serial: dict[str, int] = {}
+        self._next_serial = 0
         self.slots = StateSlots(num_state_slots)
 
     # ------------------------------------------------------------------ queries
@@ -109,6 +114,10 @@ class CacheManager:
     def num_tokens(self, request_id: str) -> int:
         return self._num_tokens[request_id]
 
+    def serial(self, request_id: str) -> int:
+        """Changes whenever ``request_id`` is allocated anew."""
+        return self._serial[request_id]
+
     def block_table(self, request_id: str, group: int = 0) -> list[int]:
         return self._tables[group][request_id]
 
@@ -127,16 +136,13 @@ class CacheManager:
             return 0
         return max(0, first_query_pos - w + 1) // self.block_size
 
-    def _new_blocks(self, g: int, table: list[int] | None, total_tokens: int, first_query_pos: int
-                    ) -> int:
-        """Pages group ``g`` must take so that positions the next queries (from
-        ``first_query_pos`` on) can see, up to ``total_tokens``, are backed."""
+    def _new_blocks(self, g: int, request_id: str | None, total_tokens: int) -> int:
+        """Pages group ``g`` must take to back positions up to ``total_tokens``.  A table only
+        grows at its end (pages a window has passed are never taken back), so this is the number
+        of entries it lacks."""
         need = self.blocks_needed(total_tokens)
-        lo = self._first_live_block(g, first_query_pos)
-        if table is None:
-            return max(0, need - lo)
-        held = sum(1 for i in range(lo, min(len(table), need)) if table[i] != RELEASED)
-        return max(0, need - lo) - held
+        have = len(self._tables[g][request_id]) if request_id is not None else 0
+        return max(0, need - have)
 
     # --------------------------------------------------------------- life cycle
     def can_allocate(self, num_tokens: int) -> bool:
@@ -144,7 +150,7 @@ class CacheManager:
         (src/tokenvault/cache/block_manager.py:165-170)."""
         if self.slots.num_slots and self.slots.num_free == 0:
             return False
-        return all(self._new_blocks(g, None, num_tokens, 0) <= p.num_free - wm
+        return all(self._new_blocks(g, None, num_tokens) <= p.num_free - wm
                    for g, (p, wm) in enumerate(zip(self.pools, self.watermark_blocks)))
 
     def allocate(self, request_id: str, num_tokens: int) -> None:
@@ -152,36 +158,40 @@ class CacheManager:
         if request_id in self._num_tokens:
             raise ValueError(f"request {request_id} already allocated")
         for g, p in enumerate(self.pools):
-            if self._new_blocks(g, None, num_tokens, 0) > p.num_free:
+            if self._new_blocks(g, None, num_tokens) > p.num_free:
                 raise NoFreeBlocksError(f"cannot allocate {num_tokens} tokens for {request_id}")
         if self.slots.num_slots:
             self.slots.take(request_id)
         for g in range(len(self.groups)):
             self._tables[g][request_id] = []
+            self._released[g][request_id] = 0
         self._num_tokens[request_id] = 0
+        self._serial[request_id] = self._next_serial
+        self._next_serial += 1
         self.append_slots(request_id, num_tokens, 0)
 
     def can_append_slots(self, request_id: str, total_tokens: int, write_start: int) -> bool:
         """Room to grow ``request_id`` to ``total_tokens`` positions, no watermark
         (src/tokenvault/cache/block_manager.py:204-207)."""
-        return all(self._new_blocks(g, self._tables[g][request_id], total_tokens, write_start)
-                   <= p.num_free for g, p in enumerate(self.pools))
+        for g, p in enumerate(self.pools):
+            if self._new_blocks(g, request_id, total_tokens) > p.num_free:
+                return False
+        return True
 
     def append_slots(self, request_id: str, total_tokens: int, write_start: int) -> None:
         """Back every position in ``[write_start, total_tokens)`` (and what those queries still
         see) with pages.  All-or-nothing: raises before taking anything if a pool is short."""
-        if not self.can_append_slots(request_id, total_tokens, write_start):
-            raise NoFreeBlocksError(f"cannot append slots for {request_id}")
         need = self.blocks_needed(total_tokens)
-        for g, p in enumerate(self.pools):
-            table = self._tables[g][request_id]
-            lo = self._first_live_block(g, write_start)
-            while len(table) < need:
-                table.append(RELEASED)
-            for i in range(lo, need):
-                if table[i] == RELEASED:
-                    table[i] = p.take()
-        self._num_tokens[request_id] = max(self._num_tokens[request_id], total_tokens)
+        short = [g for g in range(len(self.pools)) if len(self._tables[g][request_id]) < need]
+        if short:
+            if not self.can_append_slots(request_id, total_tokens, write_start):
+                raise NoFreeBlocksError(f"cannot append slots for {request_id}")
+            for g in short:
+                p, table = self.pools[g], self._tables[g][request_id]
+                while len(table) < need:
+                    table.append(p.take())
+        if total_tokens > self._num_tokens[request_id]:
+            self._num_tokens[request_id] = total_tokens
 
     def release_behind(self, request_id: str, num_computed: int) -> int:
         """Give back pages of windowed groups that no later query can see: the next query sits at
@@ -194,11 +204,14 @@ class CacheManager:
             table = self._tables[g].get(request_id)
             if table is None:
                 continue
-            for i in range(min(self._first_live_block(g, num_computed), len(table))):
+            upto = min(self._first_live_block(g, num_computed), len(table))
+            for i in range(self._released[g][request_id], upto):
                 if table[i] != RELEASED:
                     p.release(table[i])
                     table[i] = RELEASED
                     n += 1
+            if upto > self._released[g][request_id]:
+                self._released[g][request_id] = upto
         return n
 
     def free(self, request_id: str) -> None:
@@ -206,7 +219,9 @@ class CacheManager:
         (src/tokenvault/cache/block_manager.py:268-276)."""
         if self._num_tokens.pop(request_id, None) is None:
             return
+        self._serial.pop(request_id, None)
         for g, p in enumerate(self.pools):
+            self._released[g].pop(request_id, None)
             for b in reversed(self._tables[g].pop(request_id)):
                 if b != RELEASED:
                     p.release(b)

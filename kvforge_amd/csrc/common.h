@@ -18,12 +18,9 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t b) {
   return __uint_as_float(static_cast<uint32_t>(b) << 16);
 }
 
-// round to nearest even, NaN kept quiet
+// round to nearest even (the hardware conversion of gfx950)
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 template <typename T> struct Elem;
@@ -51,6 +48,22 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
     v[2 * i] = __uint_as_float(w[i] << 16);
     v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
   }
+}
+
+// Sum over aligned groups of G neighbouring lanes (G = 2..32), left in every lane of the group.
+// Data-parallel-primitive moves ride in the add itself; only the 32-lane step crosses a row
+// of 16 and needs the LDS crossbar.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int G> __device__ __forceinline__ float group_sum(float v) {
+  static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32, "group size");
+  if (G >= 2) v += dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]: lane ^ 1
+  if (G >= 4) v += dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]: lane ^ 2
+  if (G >= 8) v += dpp_move<0x141>(v);   // row_half_mirror: the other quad of 8 lanes
+  if (G >= 16) v += dpp_move<0x140>(v);  // row_mirror: the other half of 16 lanes
+  if (G >= 32) v += __shfl_xor(v, 16, KVF_WAVE);
+  return v;
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

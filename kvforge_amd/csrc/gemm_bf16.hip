@@ -7,8 +7,11 @@
 // of the same rows.  Per k-step a lane loads 16 B of W (row lane%16, k-offset 8*(lane/16)) and
 // the matching 8 elements of each 16-row tile of A and issues one v_mfma_f32_16x16x32_bf16 per
 // tile with W as the first operand, so a lane ends up holding four consecutive output columns of
-// one row of C.  Partial sums of the waves are added in wave order through LDS.  The number of
-// waves depends on N, K and on how many 16-row tiles a pass holds, never on the rows themselves.
+// one row of C.  Partial sums of the waves are added in wave order through LDS.  With several
+// row tiles of A (more than 16 rows) a wave takes NT neighbouring 16-row groups of W per k-step
+// and reuses its A fragments for them, which divides the traffic for A (served by L2) by NT.
+// The launch shape depends on N, K and on how many 16-row tiles a pass holds (1, 2, 4 or 8),
+// never on the rows themselves.
 //
 // Left operand (AT): 0 = bf16 activations; 1 = the fp32 residual stream with the RMS norm folded
 // in: y = x * rsqrt(mean(x^2) + eps) is applied as a per-row factor on the accumulators (the
@@ -46,39 +49,104 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
 
 // 8 fp32 -> 8 bf16 (round to nearest even); adds their squares to ss
 __device__ __forceinline__ bf16x8 load_frag_f32(const float* p, bool ok, float& ss) {
+  typedef __attribute__((ext_vector_type(8))) float f32x8;
   float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   if (ok) load8(p, v);
-  uint32_t w[4];
+  f32x8 x;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    ss = fmaf(v[2 * i], v[2 * i], ss);
-    ss = fmaf(v[2 * i + 1], v[2 * i + 1], ss);
-    w[i] = static_cast<uint32_t>(f32_to_bf16(v[2 * i])) |
-           (static_cast<uint32_t>(f32_to_bf16(v[2 * i + 1])) << 16);
+  for (int i = 0; i < 8; ++i) {
+    ss = fmaf(v[i], v[i], ss);
+    x[i] = v[i];
   }
-  return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+  return __builtin_convertvector(x, bf16x8);
 }
 
-// more row tiles per pass mean more registers per lane and more LDS per wave: fewer waves; fp32
+// One lane's four neighbouring columns n..n+3 of row m, after the waves' partial sums are added.
+template <int EPI>
+__device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, int ldc, void* Cv,
+                                           const RopeEpi& rp) {
+  if (EPI <= 2) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (n + r >= N) break;
+      const size_t idx = static_cast<size_t>(m) * ldc + n + r;
+      if (EPI == 0) static_cast<float*>(Cv)[idx] = s[r];
+      if (EPI == 1) static_cast<bf16_t*>(Cv)[idx].bits = f32_to_bf16(s[r]);
+      if (EPI == 2) static_cast<float*>(Cv)[idx] += s[r];
+    }
+  } else if (EPI == 3) {
+    // N is even and n a multiple of 4: two (gate, up) pairs
+    bf16_t* o = static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n / 2;
+    o[0].bits = f32_to_bf16(s[0] / (1.f + __expf(-s[0])) * s[1]);
+    if (n + 2 < N) o[1].bits = f32_to_bf16(s[2] / (1.f + __expf(-s[2])) * s[3]);
+  } else {
+    // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head
+    const int head = n / rp.d, e = n - head * rp.d;
+    const int p = rp.positions[m];
+    const bool pos_ok = p >= 0 && p < rp.table_len;
+    float o[4] = {s[0], s[1], s[2], s[3]};
+    if (head < rp.H + rp.KV && pos_ok) {
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const int j = (e + 2 * pr) / 2;
+        if (2 * j + 1 < rp.rot) {
+          const float c = rp.cos_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
+          const float sn = rp.sin_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
+          const float x1 = s[2 * pr], x2 = s[2 * pr + 1];
+          o[2 * pr] = x1 * c - x2 * sn;
+          o[2 * pr + 1] = x2 * c + x1 * sn;
+        }
+      }
+    }
+    uint2 packed;
+    packed.x = static_cast<uint32_t>(f32_to_bf16(o[0])) | (static_cast<uint32_t>(f32_to_bf16(o[1])) << 16);
+    packed.y = static_cast<uint32_t>(f32_to_bf16(o[2])) | (static_cast<uint32_t>(f32_to_bf16(o[3])) << 16);
+    if (head < rp.H) {
+      *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n) = packed;
+    } else if (rp.write_kv && pos_ok) {
+      const int seq = rp.seq_of_token[m];
+      const int blk = p / rp.block_size;
+      int page = -1;
+      if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
+        page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
+      if (page >= 0 && page < rp.num_blocks) {
+        const bool is_k = head < rp.H + rp.KV;
+        const int kvh = is_k ? head - rp.H : head - rp.H - rp.KV;
+        bf16_t* pages = is_k ? rp.k_pages : rp.v_pages;
+        *reinterpret_cast<uint2*>(
+            pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size +
+                     (p - blk * rp.block_size)) * rp.d + e) = packed;
+      }
+    }
+  }
+}
+
+// more tiles per wave mean more registers per lane and more LDS per wave: fewer waves; fp32
 // rows take twice the registers while in flight
-constexpr int max_waves(int mt, int at) {
-  return at ? (mt == 1 ? 16 : mt == 2 ? 8 : 4) : (mt <= 2 ? 16 : (mt == 4 ? 8 : 4));
+constexpr int max_waves(int mt, int nt, int at) {
+  return (mt * nt >= 8 || (at && mt >= 4)) ? 4 : (mt * nt >= 4 || (at && mt >= 2)) ? 8 : 16;
 }
 // k-steps whose loads are in flight together in one wave
-constexpr int depth(int mt, int at) { return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : 4; }
+constexpr int depth(int mt, int nt, int at) {
+  return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : (mt * nt == 1 ? 8 : mt * nt <= 4 ? 4 : 2);
+}
 
-template <int MT, int AT, int EPI>
-__global__ __launch_bounds__(max_waves(MT, AT) * KVF_WAVE) void gemm_skinny_kernel(
+template <int MT, int NT, int AT, int EPI>
+__global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
     int K, int lda, int ldc, int m_base, float eps, RopeEpi rp) {
   extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
   const int nw = blockDim.x / KVF_WAVE;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NT;
   const int r16 = lane % 16, kg = lane / 16;
-  int wrow = n0 + r16;
-  if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
-  const bf16_t* wp = W + static_cast<size_t>(wrow) * K + kg * 8;
+  const bf16_t* wp[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    int wrow = n0 + j * 16 + r16;
+    if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
+    wp[j] = W + static_cast<size_t>(wrow) * K + kg * 8;
+  }
   size_t aoff[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -88,21 +156,26 @@ __global__ __launch_bounds__(max_waves(MT, AT) * KVF_WAVE) void gemm_skinny_kern
   }
   const bf16_t* Ab = static_cast<const bf16_t*>(Av);
   const float* Af = static_cast<const float*>(Av);
-  f32x4 acc[MT];
+  f32x4 acc[NT][MT];
   float ss[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) { acc[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const int ksteps = (K + 31) / 32;
   int ks = wave;
-  constexpr int U = depth(MT, AT);
+  constexpr int U = depth(MT, NT, AT);
   for (; ks + (U - 1) * nw < ksteps; ks += U * nw) {
-    bf16x8 wf[U], af[U][MT];
+    bf16x8 wf[U][NT], af[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int k = (ks + u * nw) * 32;
       const bool ok = k + kg * 8 + 8 <= K;
-      wf[u] = load_frag(wp + k, ok);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) wf[u][j] = load_frag(wp[j] + k, ok);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         af[u][t] = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
@@ -110,137 +183,113 @@ __global__ __launch_bounds__(max_waves(MT, AT) * KVF_WAVE) void gemm_skinny_kern
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], af[u][t], acc[t], 0, 0, 0);
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][j], af[u][t], acc[j][t], 0, 0, 0);
   }
   for (; ks < ksteps; ks += nw) {
     const int k = ks * 32;
     const bool ok = k + kg * 8 + 8 <= K;
-    const bf16x8 wf = load_frag(wp + k, ok);
+    bf16x8 af[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const bf16x8 af = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af, acc[t], 0, 0, 0);
+    for (int t = 0; t < MT; ++t)
+      af[t] = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const bf16x8 wf = load_frag(wp[j] + k, ok);
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af[t], acc[j][t], 0, 0, 0);
     }
   }
-  // lane holds C[row r16][cols n0 + 4*kg .. +3] of each tile
+  // lane holds C[row r16][cols n0 + 16*j + 4*kg .. +3] of each tile
   float* red_ss = red + nw * MT * KVF_WAVE * 4;
+  if (AT) {
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * KVF_WAVE + lane) * 4) = acc[t];
-    if (AT) {
+    for (int t = 0; t < MT; ++t) {
       float v = ss[t];
       v += __shfl_xor(v, 16, KVF_WAVE);
       v += __shfl_xor(v, 32, KVF_WAVE);
       if (kg == 0) red_ss[(wave * MT + t) * 16 + r16] = v;
     }
   }
-  __syncthreads();
-  for (int item = threadIdx.x; item < MT * KVF_WAVE; item += blockDim.x) {
-    const int t = item / KVF_WAVE, l = item % KVF_WAVE;
-    f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int w = 0; w < nw; ++w)
-      s += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * KVF_WAVE + l) * 4);
-    const int m = m_base + t * 16 + l % 16;
-    const int n = n0 + 4 * (l / 16);
-    if (m >= M || n >= N) continue;
-    if (AT) {
-      float tot = 0.f;
-      for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
-      s *= rsqrtf(tot / static_cast<float>(K) + eps);
-    }
-    if (EPI <= 2) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (n + r >= N) break;
-        const size_t idx = static_cast<size_t>(m) * ldc + n + r;
-        if (EPI == 0) static_cast<float*>(Cv)[idx] = s[r];
-        if (EPI == 1) static_cast<bf16_t*>(Cv)[idx].bits = f32_to_bf16(s[r]);
-        if (EPI == 2) static_cast<float*>(Cv)[idx] += s[r];
-      }
-    } else if (EPI == 3) {
-      // N is even and n a multiple of 4: two (gate, up) pairs
-      bf16_t* o = static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n / 2;
-      o[0].bits = f32_to_bf16(s[0] / (1.f + __expf(-s[0])) * s[1]);
-      if (n + 2 < N) o[1].bits = f32_to_bf16(s[2] / (1.f + __expf(-s[2])) * s[3]);
-    } else {
-      // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head
-      const int head = n / rp.d, e = n - head * rp.d;
-      const int p = rp.positions[m];
-      const bool pos_ok = p >= 0 && p < rp.table_len;
-      float o[4] = {s[0], s[1], s[2], s[3]};
-      if (head < rp.H + rp.KV && pos_ok) {
+  for (int j = 0; j < NT; ++j) {
+    if (j > 0) __syncthreads();
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr) {
-          const int j = (e + 2 * pr) / 2;
-          if (2 * j + 1 < rp.rot) {
-            const float c = rp.cos_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
-            const float sn = rp.sin_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
-            const float x1 = s[2 * pr], x2 = s[2 * pr + 1];
-            o[2 * pr] = x1 * c - x2 * sn;
-            o[2 * pr + 1] = x2 * c + x1 * sn;
-          }
-        }
+    for (int t = 0; t < MT; ++t)
+      *reinterpret_cast<f32x4*>(red + ((wave * MT + t) * KVF_WAVE + lane) * 4) = acc[j][t];
+    __syncthreads();
+    for (int item = threadIdx.x; item < MT * KVF_WAVE; item += blockDim.x) {
+      const int t = item / KVF_WAVE, l = item % KVF_WAVE;
+      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < nw; ++w)
+        s += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * KVF_WAVE + l) * 4);
+      const int m = m_base + t * 16 + l % 16;
+      const int n = n0 + j * 16 + 4 * (l / 16);
+      if (m >= M || n >= N) continue;
+      if (AT) {
+        float tot = 0.f;
+        for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
+        s *= rsqrtf(tot / static_cast<float>(K) + eps);
       }
-      uint2 packed;
-      packed.x = static_cast<uint32_t>(f32_to_bf16(o[0])) | (static_cast<uint32_t>(f32_to_bf16(o[1])) << 16);
-      packed.y = static_cast<uint32_t>(f32_to_bf16(o[2])) | (static_cast<uint32_t>(f32_to_bf16(o[3])) << 16);
-      if (head < rp.H) {
-        *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n) = packed;
-      } else if (rp.write_kv && pos_ok) {
-        const int seq = rp.seq_of_token[m];
-        const int blk = p / rp.block_size;
-        int page = -1;
-        if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
-          page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
-        if (page >= 0 && page < rp.num_blocks) {
-          const bool is_k = head < rp.H + rp.KV;
-          const int kvh = is_k ? head - rp.H : head - rp.H - rp.KV;
-          bf16_t* pages = is_k ? rp.k_pages : rp.v_pages;
-          *reinterpret_cast<uint2*>(
-              pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size +
-                       (p - blk * rp.block_size)) * rp.d + e) = packed;
-        }
-      }
+      store_tile<EPI>(s, m, n, N, ldc, Cv, rp);
     }
   }
 }
 
 int g_waves_override = 0;
 
-// Waves per workgroup: enough workgroups x waves to keep every CU streaming, at least one
-// k-step per wave, at most 16.
-int pick_waves(int N, int K) {
-  const int tiles = (N + 15) / 16, ksteps = (K + 31) / 32;
-  int nw = g_waves_override > 0 ? g_waves_override : (4096 + tiles - 1) / tiles;
+// Waves per workgroup: enough workgroups x waves to keep every CU streaming (about 2048 waves
+// in all), at least one k-step per wave.
+int pick_waves(int groups, int K) {
+  const int ksteps = (K + 31) / 32;
+  int nw = g_waves_override > 0 ? g_waves_override : (2048 + groups - 1) / groups;
   if (nw > 16) nw = 16;
   if (nw > ksteps) nw = ksteps;
   if (nw < 1) nw = 1;
   return nw;
 }
 
-template <int MT, int AT, int EPI>
+template <int MT, int NT, int AT, int EPI>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-               int m_base, int nw, float eps, const RopeEpi& rp, hipStream_t s) {
-  if (nw > max_waves(MT, AT)) nw = max_waves(MT, AT);
-  const dim3 grid((N + 15) / 16), block(nw * KVF_WAVE);
+               int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
+  const int groups = (N + 16 * NT - 1) / (16 * NT);
+  int nw = pick_waves(groups, K);
+  if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
+  const dim3 grid(groups), block(nw * KVF_WAVE);
   const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
                      lda, ldc, m_base, eps, rp);
   return kvf_last_error();
+}
+
+// How many 16-row groups of W a wave takes: more when A has several row tiles and W has rows to
+// spare (the grid must still fill the chip).
+template <int MT, int AT, int EPI>
+int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
+              int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
+  const int tiles = (N + 15) / 16;
+  if (MT >= 2 && MT <= 4 && !AT) {
+    if (MT == 4 && tiles >= 1024)
+      return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (tiles >= 512)
+      return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+  }
+  return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
 }
 
 template <int AT, int EPI>
 int launch_rows(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
                 float eps, const RopeEpi& rp, hipStream_t s) {
-  const int nw = pick_waves(N, K);
   int err = 0;
   for (int m_base = 0; m_base < M && !err; m_base += 128) {
     const int rows = M - m_base < 128 ? M - m_base : 128;
-    if (rows <= 16) err = launch_one<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
-    else if (rows <= 32) err = launch_one<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
-    else if (rows <= 64) err = launch_one<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
-    else err = launch_one<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, nw, eps, rp, s);
+    if (rows <= 16) err = launch_nt<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    else if (rows <= 32) err = launch_nt<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    else if (rows <= 64) err = launch_nt<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    else err = launch_nt<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
   }
   return err;
 }

@@ -111,6 +111,11 @@ class MetaBuffers:
         self.staging_np = [s.numpy() for s in self.staging]
         self.events: list[torch.cuda.Event | None] = [None, None]
         self.turn = 0
+        # host mirror of the block tables: a row is rewritten only where it changed since the
+        # step before (a request that keeps its row only appends pages)
+        self.table_host = [np.full((max_seqs, w), -1, dtype=np.int32) for w in self.table_widths]
+        self.row_owner: list[list[tuple | None]] = [[None] * max_seqs for _ in self.table_widths]
+        self.row_filled = [np.zeros(max_seqs, dtype=np.int64) for _ in self.table_widths]
 
     def view(self, name: str, n: int) -> torch.Tensor:
         o = self.off[name]
@@ -176,22 +181,28 @@ class Step:
         G = H // KV
         chunks = -(-G // (4 if G <= 4 else 8))
         ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
-        # about DECODE_KEYS_PER_SPLIT keys per workgroup, so that each wave's loads are all in
-        # flight at once; at most 64 splits
-        splits = max(1, min(-(-ctx // DECODE_KEYS_PER_SPLIT), 64))
+        # Few sequences: cut the key range so that a couple of hundred workgroups pull on the
+        # cache, each with at least DECODE_KEYS_PER_SPLIT keys.  Many sequences fill the chip by
+        # themselves; their key range is cut only when it is long.
+        wgs = max(1, self.n_decode * KV * chunks)
+        splits = max(-(-256 // wgs), -(-ctx // 1024))
+        splits = max(1, min(splits, -(-ctx // DECODE_KEYS_PER_SPLIT), 64))
         if splits == 1:
             return 1, None
         acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)
         ml = self.ws.buf("decode_part_ml", (self.n_decode * H * splits * 2,), torch.float32)
-        tickets = self.ws.zeros("decode_tickets", (self.n_decode * KV * chunks,), torch.int32)
-        return splits, (acc, ml, tickets)
+        return splits, (acc, ml)
 
 
 def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], tables_of, slot_of,
-              block_size: int, pad_to: int | None = None) -> list[int]:
+              block_size: int, pad_to: int | None = None,
+              windowed_groups: Sequence[bool] | None = None, serial_of=None) -> list[int]:
     """Write the batch into ``meta`` (one host-to-device copy) and point ``step`` at it.
     ``tables_of(request_id, group) -> list[int]``; ``slot_of(request_id) -> int``.
     ``pad_to``: pad a pure-decode batch with empty sequences up to this many.
+    ``windowed_groups[g]``: group ``g`` gives pages back while a request lives, so its rows are
+    rewritten whole every step.  ``serial_of(request_id)`` tells a request id that was freed and
+    allocated again from its former self (without it rows are always rewritten whole).
     Returns how many logits rows each entry gets."""
     B = len(entries)
     q_lens = [len(e.token_ids) for e in entries]
@@ -249,15 +260,29 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
 
     end = off["logits_rows"] + max(R, 1)
     for g, (to, w) in enumerate(zip(meta.table_off, meta.table_widths)):
-        tab = host[to:to + Bp * w].reshape(Bp, w)
-        tab[:] = -1
+        mirror, owner, filled = meta.table_host[g], meta.row_owner[g], meta.row_filled[g]
+        windowed = windowed_groups is not None and windowed_groups[g]
         for b, e in enumerate(entries):
             t = tables_of(e.request_id, g)
             need = -(-int(ctx[b]) // block_size)
             if need > w or need > len(t):
                 raise ValueError(f"request {e.request_id} needs {need} pages in group {g}; "
                                  f"table holds {len(t)}, width {w}")
-            tab[b, :need] = t[:need]
+            have = int(filled[b])
+            tag = (e.request_id, serial_of(e.request_id)) if serial_of is not None else None
+            if tag is not None and owner[b] == tag and have <= need and not windowed:
+                if have < need:
+                    mirror[b, have:need] = t[have:need]
+            else:
+                mirror[b, :have] = -1
+                mirror[b, :need] = t[:need]
+                owner[b] = tag
+            filled[b] = need
+        for b in range(B, Bp):
+            if filled[b]:
+                mirror[b, :int(filled[b])] = -1
+            owner[b], filled[b] = None, 0
+        host[to:to + Bp * w].reshape(Bp, w)[:] = mirror[:Bp]
         end = to + Bp * w
     meta.device_buf[:end].copy_(meta.staging[turn][:end], non_blocking=True)
     if meta.device_buf.is_cuda:

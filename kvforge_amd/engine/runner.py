@@ -49,6 +49,7 @@ class ModelRunner:
         self.meta = MetaBuffers(max(max_num_batched_tokens, max_num_seqs), max_num_seqs,
                                 [width] * len(groups), self.device)
         self.ws = Workspace(self.device)
+        self._windowed = [g.window is not None for g in groups]
         self.num_forward_passes = 0
         self.num_tokens_processed = 0
         # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph
@@ -60,6 +61,10 @@ class ModelRunner:
         self._sample_i = torch.zeros(2 * cap, dtype=torch.int32, device=self.device)
         self._sample_f_host = torch.zeros(3 * cap, dtype=torch.float32, pin_memory=True)
         self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
+        self._sample_f_np, self._sample_i_np = self._sample_f_host.numpy(), self._sample_i_host.numpy()
+        self._sample_ids: list[str] = []
+        self._sample_bucket = 0
+        self._sample_drawn: list[int] = []
 
     @staticmethod
     def bytes_per_block(model: Transformer, block_size: int) -> int:
@@ -77,7 +82,7 @@ class ModelRunner:
         step = Step()
         step.ws, step.act_dtype, step.device = self.ws, self.model.dtype, self.device
         counts = fill_step(step, self.meta, entries, self.cache.block_table, self._slot_of,
-                           self.block_size, pad_to)
+                           self.block_size, pad_to, self._windowed, self.cache.serial)
         return step, counts
 
     @torch.inference_mode()
@@ -119,17 +124,26 @@ class ModelRunner:
             ctx_bucket *= 2
         step.max_decode_ctx = ctx_bucket
         cap = self.meta.max_seqs
-        fh, ih = self._sample_f_host, self._sample_i_host
-        fh[:bucket] = 0.0                     # padding rows are greedy
-        fh[cap:cap + bucket] = 1.0
-        ih[:bucket] = 0
-        for i, (p, s, c) in enumerate(zip(params, streams, counters)):
-            fh[i] = p.temperature
-            fh[cap + i] = p.top_p
-            ih[i] = p.top_k
-            fh[2 * cap + i] = 0.0 if p.greedy else uniform(seed, s, c)
-        self._sample_f.copy_(fh, non_blocking=True)
-        self._sample_i[:cap].copy_(ih, non_blocking=True)
+        fh, ih = self._sample_f_np, self._sample_i_np
+        ids = [e.request_id for e in entries]
+        if ids != self._sample_ids or bucket != self._sample_bucket:
+            # the batch changed: rewrite the per-row parameters (padding rows are greedy)
+            fh[:bucket] = 0.0
+            fh[cap:cap + bucket] = 1.0
+            fh[2 * cap:2 * cap + bucket] = 0.0
+            ih[:bucket] = 0
+            for i, p in enumerate(params):
+                fh[i], fh[cap + i], ih[i] = p.temperature, p.top_p, p.top_k
+            self._sample_ids, self._sample_bucket = ids, bucket
+            self._sample_drawn = [i for i, p in enumerate(params) if not p.greedy]
+            self._sample_i[:cap].copy_(self._sample_i_host, non_blocking=True)
+            dirty = True
+        else:
+            dirty = bool(self._sample_drawn)
+        for i in self._sample_drawn:
+            fh[2 * cap + i] = uniform(seed, streams[i], counters[i])
+        if dirty:
+            self._sample_f.copy_(self._sample_f_host, non_blocking=True)
         key = (bucket, ctx_bucket)
         graph = self.graphs.get(key)
         if graph is None:

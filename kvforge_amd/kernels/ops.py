@@ -163,6 +163,7 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 # ------------------------------------------------------------------------------ matrix products
 # Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.
 SKINNY_MAX_M = 128
+FUSED_NORM_MAX_M = 16
 _GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
 
 
@@ -186,11 +187,13 @@ def _gemm_operands(a, w, out, n_out):
 
 def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False) -> bool:
     """Whether the MFMA weight-streaming kernel takes these operands: bf16 weights, bf16 rows
-    (or, with ``rms``, fp32 rows), 16-byte aligned rows, at most ``SKINNY_MAX_M`` of them."""
+    (or, with ``rms``, fp32 rows), 16-byte aligned rows, at most ``SKINNY_MAX_M`` of them.
+    Folding the norm in pays only while every workgroup converts one tile of rows
+    (``FUSED_NORM_MAX_M``); beyond that a norm kernel of its own is cheaper."""
     m, k = a.shape
     lda = a.stride(0) if m > 1 else k
     return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and k % 8 == 0 and lda % 8 == 0
-            and m <= SKINNY_MAX_M)
+            and m <= (FUSED_NORM_MAX_M if rms else SKINNY_MAX_M))
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -361,27 +364,23 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
             raise KernelError("attn_decode: seq_ids shorter than num_seqs")
     elif num_seqs > n_seqs:
         raise KernelError("attn_decode: more sequences than block-table rows")
-    pa = pm = tk = None
+    pa = pm = None
     if splits > 1:
         if workspace is None:
             raise KernelError("attn_decode: splits > 1 need a workspace")
-        pa, pm, tk = workspace
+        pa, pm = workspace[0], workspace[1]
         _check(pa, "workspace[0]", F32)
         _check(pm, "workspace[1]", F32)
-        _check(tk, "workspace[2]", I32)
-        G = H // KV
-        chunks = -(-G // (4 if G <= 4 else 8))
-        if (pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2
-                or tk.numel() < num_seqs * KV * chunks):
+        if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
             raise KernelError("attn_decode: workspace too small")
     nb, _, bs, _ = k_pages.shape
     f = _fn("attn_decode", "kvf_attn_decode",
-            [c_int] + [c_void_p] * 11 + [c_int] * 12 + [c_float, c_void_p])
+            [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
           cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
           pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
-          tk.data_ptr() if tk is not None else None, num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
+          num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
           int(window), n_seqs, int(splits), float(scale), _stream()), "attn_decode")
 
 

@@ -98,6 +98,11 @@ class PagedAttention(Mixer):
         table = step.block_tables[layer.group]
         cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else step.no_rotation()
         rms = self.norm_eps
+        if rms is not None and not ops.bf16_kernel_takes(x, self.w_qkv, True):
+            # too many rows for the norm to ride in the projection: a norm kernel of its own
+            normed = ws.buf("normed", (n, self.hidden), act)
+            ops.rmsnorm(x, None, rms, normed)
+            x, rms = normed, None
         if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None) and layer.k_pages.dtype == torch.bfloat16:
             # one kernel: (norm,) projection, rotary, cache write
             qkv = ws.buf("q_rot", (n, H * d), act)
@@ -105,10 +110,6 @@ class PagedAttention(Mixer):
                               layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache,
                               rms_eps=rms)
         else:
-            if rms is not None:
-                normed = ws.buf("normed", (n, self.hidden), act)
-                ops.rmsnorm(x, None, rms, normed)
-                x = normed
             qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), act)
             ops.gemm(x, self.w_qkv, qkv)
             ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,

@@ -56,14 +56,15 @@ class SwiGLU(FeedForward):
         n = x.shape[0]
         ws, dt, rms = step.ws, step.act_dtype, self.norm_eps
         act = ws.buf("ffn_act", (n, self.inter), dt)
+        if rms is not None and not ops.bf16_kernel_takes(x, self.w_gate_up, True):
+            # too many rows for the norm to ride in the projection: a norm kernel of its own
+            normed = ws.buf("normed", (n, self.hidden), dt)
+            ops.rmsnorm(x, None, rms, normed)
+            x, rms = normed, None
         if ops.bf16_kernel_takes(x, self.w_gate_up, rms is not None) and self.inter % 2 == 0:
             # one kernel: (norm,) gate/up projection, SwiGLU gate
             ops.gemm_fused(x, self.w_gate_up, act, rms_eps=rms, silu_pairs=True)
         else:
-            if rms is not None:
-                normed = ws.buf("normed", (n, self.hidden), dt)
-                ops.rmsnorm(x, None, rms, normed)
-                x = normed
             gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
             ops.gemm(x, self.w_gate_up, gu)
             ops.silu_mul(gu, act, paired=True)

@@ -141,16 +141,21 @@ def test_gemm_fused_norm_and_gate(m, n, k):
     xn = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
     want = xn.double() @ w.double().T
     out = torch.empty(m, n, device=DEV)
-    ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
-    torch.testing.assert_close(out.double().cpu(), want, atol=2e-2, rtol=2e-2)   # rows are rounded to bf16
-    res = torch.randn(m, n, generator=g)
-    acc = res.clone().to(DEV)
-    ops().gemm_fused(x.to(DEV), w.to(DEV), acc, rms_eps=eps, accumulate=True)
-    torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=2e-2, rtol=2e-2)
     gate = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
-    ops().gemm_fused(x.to(DEV), w.to(DEV), gate, rms_eps=eps, silu_pairs=True)
-    want_gate = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
-    torch.testing.assert_close(gate.double().cpu(), want_gate, atol=2e-2, rtol=3e-2)
+    if m <= ops().FUSED_NORM_MAX_M:
+        ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
+        torch.testing.assert_close(out.double().cpu(), want, atol=2e-2, rtol=2e-2)   # rows are rounded to bf16
+        res = torch.randn(m, n, generator=g)
+        acc = res.clone().to(DEV)
+        ops().gemm_fused(x.to(DEV), w.to(DEV), acc, rms_eps=eps, accumulate=True)
+        torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=2e-2, rtol=2e-2)
+        ops().gemm_fused(x.to(DEV), w.to(DEV), gate, rms_eps=eps, silu_pairs=True)
+        want_gate = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+        torch.testing.assert_close(gate.double().cpu(), want_gate, atol=2e-2, rtol=3e-2)
+    else:
+        assert not ops().bf16_kernel_takes(x.to(DEV), w.to(DEV), rms=True)
+        with pytest.raises(ops().KernelError):
+            ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
     xb = xn.to(torch.bfloat16)
     ops().gemm_fused(xb.to(DEV), w.to(DEV), gate, silu_pairs=True)
     wantb = xb.double() @ w.double().T
@@ -180,6 +185,8 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     cos_full, sin_full = plain.rope_cos_sin(torch.arange(64), inv_freq)
     cos_t, sin_t = cos_full[:, : rot // 2].contiguous().to(DEV), sin_full[:, : rot // 2].contiguous().to(DEV)
     eps = 1e-5
+    if rms and m > ops().FUSED_NORM_MAX_M:
+        pytest.skip("the norm rides in the projection only for one tile of rows")
     if rms:
         a = x.to(DEV)
         normed = torch.empty(m, k, dtype=torch.bfloat16, device=DEV)
@@ -353,7 +360,6 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     got = out2.float().cpu()
     torch.testing.assert_close(got[[4, 1]], want[[4, 1]], **tol(dtype))
     assert (got[[0, 2, 3, 5]] == 5.0).all()
-    assert int(ws[2].abs().sum()) == 0          # the tickets are left at zero
 
 
 def test_attn_far_key_stands_out():
