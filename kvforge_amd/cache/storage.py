@@ -1,7 +1,10 @@
-"""Device storage behind the cache manager: K and V pages per cache-owning layer, laid out
-``[num_blocks, kv_heads, block_size, head_dim]`` so that one (page, head) tile is contiguous, and
-state tensors ``[num_slots, *shape]`` for mixers with fixed-size state.  The reference keeps
-``[num_blocks, block_size, kv_heads, head_dim]`` per layer (src/tokenvault/cache/kv_cache.py:27-31).
+"""Device storage behind the cache manager: K and V pages per cache-owning call, and state
+tensors ``[num_slots, *shape]`` for mixers with fixed-size state.  K pages are
+``[num_blocks, kv_heads, block_size, head_dim]`` (one (page, head) tile is contiguous, a key's
+elements side by side); V pages are transposed, ``[num_blocks, kv_heads, head_dim, block_size]``
+(an element's keys side by side), which is the order the matrix cores contract ``P * V`` in.
+The reference keeps ``[num_blocks, block_size, kv_heads, head_dim]`` for both
+(src/tokenvault/cache/kv_cache.py:27-31).
 """
 
 from __future__ import annotations
@@ -20,10 +23,11 @@ class PagedStorage:
         self.v: dict[int, torch.Tensor] = {}
         self.group_of: dict[int, int] = {}
         for g, (grp, nb) in enumerate(zip(groups, num_blocks)):
-            shape = (nb, grp.num_kv_heads, block_size, grp.head_dim)
+            k_shape = (nb, grp.num_kv_heads, block_size, grp.head_dim)
+            v_shape = (nb, grp.num_kv_heads, grp.head_dim, block_size)
             for layer in grp.layers:
-                self.k[layer] = torch.zeros(shape, dtype=dtype, device=device)
-                self.v[layer] = torch.zeros(shape, dtype=dtype, device=device)
+                self.k[layer] = torch.zeros(k_shape, dtype=dtype, device=device)
+                self.v[layer] = torch.zeros(v_shape, dtype=dtype, device=device)
                 self.group_of[layer] = g
 
     @property

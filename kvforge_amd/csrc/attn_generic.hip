@@ -8,8 +8,8 @@
 // per row (all fp32).  Key j is visible to the query at position p iff j <= p, j < context
 // length and, with a window w > 0, j > p - w.  Scores are scaled after the dot product.
 //
-// Pages are [num_blocks, KV, block_size, d]; a key whose page entry is negative or out of
-// range contributes nothing.
+// K pages are [num_blocks, KV, block_size, d], V pages are transposed [num_blocks, KV, d,
+// block_size]; a key whose page entry is negative or out of range contributes nothing.
 #include "common.h"
 
 namespace {
@@ -17,6 +17,8 @@ constexpr int ROWS = 16;
 
 struct AttnArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs;
+  int tiles_per_seq;  // 0: `work` holds (sequence, tile) pairs; > 0: `work` lists sequences (or
+                      // is null for 0, 1, 2, ...) and each takes this many tiles
   float scale;
 };
 
@@ -30,7 +32,15 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   __shared__ float KVs[BKEYS][DMAX + 1];
   __shared__ float Ps[ROWS][BKEYS + 1];
 
-  const int seq = work[2 * blockIdx.x], tile = work[2 * blockIdx.x + 1];
+  int seq, tile;
+  if (a.tiles_per_seq > 0) {
+    const int idx = blockIdx.x / a.tiles_per_seq;
+    seq = work ? work[idx] : idx;
+    tile = blockIdx.x - idx * a.tiles_per_seq;
+  } else {
+    seq = work[2 * blockIdx.x];
+    tile = work[2 * blockIdx.x + 1];
+  }
   if (seq < 0 || seq >= a.n_seqs) return;
   const int kvh = blockIdx.y;
   const int G = a.H / a.KV, D = a.d;
@@ -133,21 +143,21 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
     m_run = m_new;
 #pragma unroll
     for (int j = 0; j < DMAX / 16; ++j) acc[j] *= corr;
-    // ---- V tile (overwrites the K tile once every thread has finished with it)
+    // ---- V tile (overwrites the K tile once every thread has finished with it); V pages hold
+    // the keys of one element side by side, so a thread walks keys fastest
     __syncthreads();
-    for (int ch = tid; ch < BKEYS * chunks_per_key; ch += 256) {
-      const int c = ch / chunks_per_key, k8 = (ch - c * chunks_per_key) * 8;
+    for (int idx = tid; idx < BKEYS * D; idx += 256) {
+      const int e = idx / BKEYS, c = idx - e * BKEYS;
       const int j = t0 + c;
-      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      float v = 0.f;
       if (j >= lo && j <= hi) {
         const int blk = j / a.block_size;
         const int page = blk < a.table_stride ? table[blk] : -1;
         if (page >= 0 && page < a.num_blocks)
-          load8(v_pages + ((static_cast<size_t>(page) * a.KV + kvh) * a.block_size +
-                           (j - blk * a.block_size)) * D + k8, v);
+          v = Elem<T>::load(v_pages + ((static_cast<size_t>(page) * a.KV + kvh) * D + e) * a.block_size +
+                            (j - blk * a.block_size));
       }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) KVs[c][k8 + e] = v[e];
+      KVs[c][e] = v;
     }
     __syncthreads();
     for (int c = 0; c < BKEYS; ++c) {
@@ -186,17 +196,21 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
 }  // namespace
 
 // dtype: 0 = fp32, 1 = bf16.  d must be a multiple of 16 and at most 256 (checked by the caller
-// and here).  `work` holds num_work pairs (sequence, 16-row tile).
+// and here).  tiles_per_seq == 0: `work` holds num_work pairs (sequence, 16-row tile).
+// tiles_per_seq > 0: num_work sequences, listed in `work` or 0..num_work-1 when it is null, each
+// with that many tiles (single-token queries need ceil(G / 16)).
 KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, const void* v_pages,
                                 const int* block_table, const int* cu_q, const int* ctx_lens,
-                                const int* work, int num_work, void* out, int H, int KV, int d,
-                                int block_size, int num_blocks, int table_stride, int q_stride,
-                                int o_stride, int window, int n_seqs, float scale,
+                                const int* work, int num_work, int tiles_per_seq, void* out, int H,
+                                int KV, int d, int block_size, int num_blocks, int table_stride,
+                                int q_stride, int o_stride, int window, int n_seqs, float scale,
                                 hipStream_t s) {
-  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0)
+  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || tiles_per_seq < 0 ||
+      (tiles_per_seq == 0 && !work))
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             scale};
+             tiles_per_seq, scale};
+  if (tiles_per_seq > 0) num_work *= tiles_per_seq;
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)

@@ -131,7 +131,9 @@ KVF_EXPORT int kvf_silu_mul_bf16(const void* gu, void* out, int m, int inter, in
 // elements at or beyond `rot` are copied.  q is rotated in place.
 // Rotated k and v go to the pages: page = block_table[seq_of_token[n], p / block_size];
 // a negative page (padding, or a page already given back) or p outside the table skips the write.
-// Pages are [num_blocks, KV, block_size, d].  With write_kv == 0 only q is rotated.
+// K pages are [num_blocks, KV, block_size, d]; V pages are transposed, [num_blocks, KV, d,
+// block_size], so that the keys of one element lie side by side (what the P*V product of the
+// matrix cores contracts over).  With write_kv == 0 only q is rotated.
 struct RopeArgs {
   int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
 };
@@ -189,8 +191,8 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
   }
   for (int t = threadIdx.x; t < a.KV * a.d; t += blockDim.x) {
     const int hh = t / a.d, i = t - hh * a.d;
-    T* dst = v_pages + ((static_cast<size_t>(page) * a.KV + hh) * a.block_size + off) * a.d;
-    dst[i] = row[(a.H + a.KV + hh) * a.d + i];
+    v_pages[((static_cast<size_t>(page) * a.KV + hh) * a.d + i) * a.block_size + off] =
+        row[(a.H + a.KV + hh) * a.d + i];
   }
 }
 

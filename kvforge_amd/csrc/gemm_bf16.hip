@@ -22,7 +22,8 @@
 // 3 SwiGLU gate: columns come in (gate, up) pairs, out[m, j] = silu(c[2j]) * c[2j+1] as bf16;
 // 4 rotary + cache write for a fused q/k/v projection: neighbouring columns of q and k heads are
 //   rotary pairs; rotated q goes to the output (bf16, q heads only), rotated k and plain v go
-//   straight into the pages of the token's sequence.
+//   straight into the pages of the token's sequence (K pages [nb, KV, block, d], V pages
+//   transposed [nb, KV, d, block]).
 // K must be a multiple of 8 (16-byte loads); a k-step that passes K loads zeros.
 #include "common.h"
 
@@ -110,12 +111,20 @@ __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, 
       if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
         page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
       if (page >= 0 && page < rp.num_blocks) {
-        const bool is_k = head < rp.H + rp.KV;
-        const int kvh = is_k ? head - rp.H : head - rp.H - rp.KV;
-        bf16_t* pages = is_k ? rp.k_pages : rp.v_pages;
-        *reinterpret_cast<uint2*>(
-            pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size +
-                     (p - blk * rp.block_size)) * rp.d + e) = packed;
+        const int off = p - blk * rp.block_size;
+        if (head < rp.H + rp.KV) {
+          const int kvh = head - rp.H;
+          *reinterpret_cast<uint2*>(
+              rp.k_pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size + off) * rp.d +
+              e) = packed;
+        } else {
+          // V pages are [num_blocks, KV, d, block_size]: one element per key row
+          const int kvh = head - rp.H - rp.KV;
+          bf16_t* dst = rp.v_pages +
+                        ((static_cast<size_t>(page) * rp.KV + kvh) * rp.d + e) * rp.block_size + off;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) dst[static_cast<size_t>(r) * rp.block_size].bits = f32_to_bf16(o[r]);
+        }
       }
     }
   }

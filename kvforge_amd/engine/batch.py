@@ -149,21 +149,24 @@ class Step:
         self.prefill_seqs: list[int] = []
         self.max_decode_ctx = 0
         self.max_position = 0
-        self._work: dict[int, torch.Tensor | None] = {}
+        self._work: dict[tuple[int, int], torch.Tensor | None] = {}
         self._identity_rotary = None
         self.device: torch.device | str = "cuda"
 
-    def prefill_work(self, group_size: int) -> torch.Tensor | None:
-        """``[num_work, 2]`` (sequence row, 16-row tile) for every query run longer than one
-        token, given ``group_size`` query heads per kv head."""
+    def prefill_work(self, group_size: int, rows_per_item: int = ROWS_PER_TILE
+                     ) -> torch.Tensor | None:
+        """``[num_work, 2]`` (sequence row, item) for every query run longer than one token: a
+        run of ``q`` tokens has ``q * group_size`` rows per kv head, an item covers
+        ``rows_per_item`` of them."""
         if not self.prefill_seqs:
             return None
-        w = self._work.get(group_size)
+        key = (group_size, rows_per_item)
+        w = self._work.get(key)
         if w is None:
             pairs = [(b, t) for b in self.prefill_seqs
-                     for t in range(-(-self.q_lens[b] * group_size // ROWS_PER_TILE))]
+                     for t in range(-(-self.q_lens[b] * group_size // rows_per_item))]
             w = torch.tensor(pairs, dtype=torch.int32).reshape(-1, 2).to(self.device)
-            self._work[group_size] = w
+            self._work[key] = w
         return w
 
     def no_rotation(self) -> tuple[torch.Tensor, torch.Tensor]:
@@ -179,7 +182,7 @@ class Step:
     def decode_plan(self, H: int, KV: int, d: int, window: int):
         """How many splits of the key range the decode kernel uses, and its workspace."""
         G = H // KV
-        chunks = -(-G // (4 if G <= 4 else 8))
+        chunks = -(-G // 16)
         ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
         # Few sequences: cut the key range so that a couple of hundred workgroups pull on the
         # cache, each with at least DECODE_KEYS_PER_SPLIT keys.  Many sequences fill the chip by

@@ -32,8 +32,7 @@ MODULES: dict[str, list[str]] = {
     "gemm_generic": ["gemm_generic.hip"],
     "gemm_bf16": ["gemm_bf16.hip"],
     "attn_generic": ["attn_generic.hip"],
-    "attn_decode": ["attn_decode.hip"],
-    "attn_prefill_bf16": ["attn_prefill_bf16.hip"],
+    "attn_mfma": ["attn_mfma.hip"],
     "sampling": ["sampling.hip"],
 }
 

@@ -133,7 +133,8 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
                  head_dim: int, write_kv: bool = True) -> None:
     """Rotate q (in place) and k by the cos/sin rows of each token's position; write rotated k
     and v into the pages named by the token's sequence row of ``block_table``.  Rotary pairs
-    are neighbouring elements ``(2i, 2i + 1)`` of a head."""
+    are neighbouring elements ``(2i, 2i + 1)`` of a head.  ``k_pages``:
+    ``[num_blocks, KV, block_size, d]``; ``v_pages`` transposed: ``[num_blocks, KV, d, block_size]``."""
     n = qkv.shape[0]
     H, KV, d = num_heads, num_kv_heads, head_dim
     _check(qkv, "qkv", None, (n, (H + 2 * KV) * d))
@@ -150,8 +151,8 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
     _check(block_table, "block_table", I32, (None, None))
     n_seqs, stride = block_table.shape
     _check(k_pages, "k_pages", qkv.dtype, (None, KV, None, d))
-    _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
     nb, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", qkv.dtype, (nb, KV, d, bs))
     f = _fn("elementwise", f"kvf_rope_kvwrite_{_suffix(qkv.dtype)}",
             [c_void_p] * 8 + [c_int] * 11 + [c_void_p])
     _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(),
@@ -285,8 +286,8 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
         raise KernelError(f"gemm_qkv_rope: rotary width {2 * half} / head_dim {d} not supported")
     _check(block_table, "block_table", I32, (None, None))
     _check(k_pages, "k_pages", BF16, (None, KV, None, d))
-    _check(v_pages, "v_pages", BF16, tuple(k_pages.shape))
     nb, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", BF16, (nb, KV, d, bs))
     if m == 0:
         return
     f = _fn("gemm_bf16", "kvf_gemm_bf16_qkv_rope",
@@ -318,7 +319,8 @@ def _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d
     if q.stride(1) != 1 or q.shape[1] < H * d:
         raise KernelError("attention: q rows must be dense and hold all query heads")
     _check(k_pages, "k_pages", q.dtype, (None, KV, None, d))
-    _check(v_pages, "v_pages", q.dtype, tuple(k_pages.shape))
+    nb, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", q.dtype, (nb, KV, d, bs))
     _check(block_table, "block_table", I32, (None, None))
     n_seqs = block_table.shape[0]
     _check(cu_q, "cu_q", I32, (None,))
@@ -331,22 +333,54 @@ def _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d
     return n_seqs
 
 
+def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
+    """The MFMA attention kernels take bf16 and pages of a multiple of 8 tokens; everything else
+    (the true 32-bit path above all) runs the vector-ALU kernel."""
+    return dtype == BF16 and block_size % 8 == 0
+
+
+def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int) -> int:
+    """Rows of (query token, head in group) that one entry of a prefill work list covers."""
+    if attention_on_matrix_cores(dtype, block_size):
+        return 128 if head_dim <= 128 else 64
+    return 16
+
+
 def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
-                 head_dim: int, scale: float, window: int = 0, force_generic: bool = False) -> None:
+                 head_dim: int, scale: float, window: int = 0) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 2]`` pairs
-    (sequence row, tile of 16 rows) where a sequence has ``query_len * H/KV`` rows per kv head."""
+    (sequence row, item) where a sequence has ``query_len * H/KV`` rows per kv head and an item
+    covers ``prefill_rows_per_item(...)`` of them.  ``v_pages`` are transposed:
+    ``[num_blocks, KV, head_dim, block_size]``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     _check(work, "work", I32, (None, 2))
     nb, _, bs, _ = k_pages.shape
+    if attention_on_matrix_cores(q.dtype, bs):
+        f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
+                [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p])
+        _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
+              cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], out.data_ptr(),
+              H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window),
+              n_seqs, float(scale), _stream()), "attn_mfma_prefill")
+        return
+    _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, work.shape[0], 0, out,
+                  H, KV, d, scale, window, n_seqs)
+
+
+def _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, tiles_per_seq,
+                  out, H, KV, d, scale, window, n_seqs) -> None:
+    nb, _, bs, _ = k_pages.shape
     f = _fn("attn_generic", "kvf_attn_generic",
-            [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p])
+            [c_int] + [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 10
+            + [c_float, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-          block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
-          work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
-          out.stride(0), int(window), n_seqs, float(scale), _stream()), "attn_generic")
+          block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(),
+          work.data_ptr() if work is not None else None, num_work, tiles_per_seq, out.data_ptr(),
+          H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs,
+          float(scale), _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -355,7 +389,9 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
-    each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys."""
+    each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  On the
+    matrix cores the key range may be cut into ``splits`` runs; ``workspace`` then holds fp32
+    partial accumulators and fp32 (max, sum) pairs.  The vector-ALU kernel ignores ``splits``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     if seq_ids is not None:
@@ -364,6 +400,11 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
             raise KernelError("attn_decode: seq_ids shorter than num_seqs")
     elif num_seqs > n_seqs:
         raise KernelError("attn_decode: more sequences than block-table rows")
+    nb, _, bs, _ = k_pages.shape
+    if not attention_on_matrix_cores(q.dtype, bs):
+        _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, seq_ids, num_seqs,
+                      -(-(H // KV) // 16), out, H, KV, d, scale, window, n_seqs)
+        return
     pa = pm = None
     if splits > 1:
         if workspace is None:
@@ -373,15 +414,14 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         _check(pm, "workspace[1]", F32)
         if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
             raise KernelError("attn_decode: workspace too small")
-    nb, _, bs, _ = k_pages.shape
-    f = _fn("attn_decode", "kvf_attn_decode",
-            [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
-    _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-          block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
-          cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
-          pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
-          num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
-          int(window), n_seqs, int(splits), float(scale), _stream()), "attn_decode")
+    f = _fn("attn_mfma", "kvf_attn_mfma_decode",
+            [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+    _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
+          seq_ids.data_ptr() if seq_ids is not None else None, cu_q.data_ptr(),
+          ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
+          pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
+          block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs, int(splits),
+          float(scale), _stream()), "attn_mfma_decode")
 
 
 # ------------------------------------------------------------------------------ sampling

@@ -81,9 +81,9 @@ class PagedAttention(Mixer):
         return True
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
-        mods = {"elementwise", "gemm_generic", "attn_generic", "attn_decode"}
+        mods = {"elementwise", "gemm_generic", "attn_generic"}
         if dtype == torch.bfloat16:
-            mods |= {"gemm_bf16"}
+            mods |= {"gemm_bf16", "attn_mfma"}
         return mods
 
     def num_bytes(self) -> int:
@@ -116,7 +116,8 @@ class PagedAttention(Mixer):
                              layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache)
         out = ws.buf("attn_out", (n, H * d), act)
         window = self.window or 0
-        work = step.prefill_work(H // KV)
+        bs = layer.k_pages.shape[2]
+        work = step.prefill_work(H // KV, ops.prefill_rows_per_item(act, d, bs))
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window)

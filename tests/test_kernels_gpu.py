@@ -198,10 +198,10 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     qkv = torch.empty(m, (H + 2 * KV) * d, dtype=torch.bfloat16, device=DEV)
     ops().gemm(ref_in, w, qkv)
     kp_ref = torch.zeros(nb, KV, bs, d, dtype=torch.bfloat16, device=DEV)
-    vp_ref = torch.zeros_like(kp_ref)
+    vp_ref = torch.zeros(nb, KV, d, bs, dtype=torch.bfloat16, device=DEV)
     ops().rope_kvwrite(qkv, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV), kp_ref,
                        vp_ref, H, KV, d)
-    kp, vp = torch.zeros_like(kp_ref), torch.zeros_like(kp_ref)
+    kp, vp = torch.zeros_like(kp_ref), torch.zeros_like(vp_ref)
     q = torch.empty(m, H * d, dtype=torch.bfloat16, device=DEV)
     ops().gemm_qkv_rope(a, w, q, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV), kp,
                         vp, H, KV, d, rms_eps=eps if rms else None)
@@ -220,7 +220,8 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
             once[page, pos % bs] = True
     sel = once[:, None, :, None].expand(nb, KV, bs, d)
     torch.testing.assert_close(kp.float().cpu()[sel], kp_ref.float().cpu()[sel], **t)
-    torch.testing.assert_close(vp.float().cpu()[sel], vp_ref.float().cpu()[sel], **t)
+    sel_v = once[:, None, None, :].expand(nb, KV, d, bs)
+    torch.testing.assert_close(vp.float().cpu()[sel_v], vp_ref.float().cpu()[sel_v], **t)
     assert once.any()
     untouched = (kp_ref.float().cpu().abs().sum((1, 3)) == 0)
     assert (kp.float().cpu().abs().sum((1, 3))[untouched] == 0).all()
@@ -250,7 +251,8 @@ def test_gemm_rows_do_not_depend_on_batch():
 
 
 class Paged:
-    """Scatters contiguous per-sequence K/V into shuffled pages ``[nb, KV, bs, d]``."""
+    """Scatters contiguous per-sequence K/V into shuffled pages: K ``[nb, KV, bs, d]``, V
+    transposed ``[nb, KV, d, bs]``."""
 
     def __init__(self, seq_lens, KV, d, bs, dtype, seed=0, spare=7):
         rng = random.Random(seed)
@@ -260,7 +262,7 @@ class Paged:
         ids = list(range(self.nb))
         rng.shuffle(ids)
         self.k = torch.randn(self.nb, KV, bs, d, generator=g).to(dtype)  # junk everywhere
-        self.v = torch.randn(self.nb, KV, bs, d, generator=g).to(dtype)
+        self.v = torch.randn(self.nb, KV, d, bs, generator=g).to(dtype)
         width = max(-(-n // bs) for n in seq_lens) + 2
         self.table = torch.full((len(seq_lens), width), -1, dtype=torch.int32)
         self.keys, self.values = [], []
@@ -273,7 +275,7 @@ class Paged:
                 seg = slice(b * bs, min(n, (b + 1) * bs))
                 cnt = seg.stop - seg.start
                 self.k[page, :, :cnt] = kk[seg].transpose(0, 1)
-                self.v[page, :, :cnt] = vv[seg].transpose(0, 1)
+                self.v[page, :, :, :cnt] = vv[seg].permute(1, 2, 0)
             self.keys.append(kk)
             self.values.append(vv)
 
@@ -287,10 +289,11 @@ def attn_reference(paged, q, seq_lens, q_lens, scale, window):
     return torch.cat(outs)
 
 
-def prefill_work(q_lens, G):
+def prefill_work(q_lens, G, dtype=torch.float32, d=16, bs=4):
+    rows = ops().prefill_rows_per_item(dtype, d, bs)
     work = []
     for s, ql in enumerate(q_lens):
-        for t in range(-(-ql * G // 16)):
+        for t in range(-(-ql * G // rows)):
             work.append((s, t))
     return torch.tensor(work, dtype=torch.int32).reshape(-1, 2)
 
@@ -307,7 +310,8 @@ ATTN_CASES = [
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("seq_lens,q_lens", ATTN_CASES)
 @pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
-                                        (4, 4, 80, 16), (8, 2, 128, 16), (2, 1, 256, 32)])
+                                        (4, 4, 80, 16), (8, 2, 128, 16), (2, 1, 256, 32),
+                                        (32, 8, 64, 16), (20, 1, 16, 8)])
 @pytest.mark.parametrize("window", [0, 11])
 def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
     paged = Paged(seq_lens, KV, d, bs, dtype, seed=len(seq_lens) + d)
@@ -321,7 +325,7 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
     out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
     scale = 1 / math.sqrt(d)
     ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
-                       cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV).to(DEV), out,
+                       cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV, dtype, d, bs).to(DEV), out,
                        H, KV, d, scale, window)
     want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
@@ -330,7 +334,7 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
                                         (4, 4, 80, 16), (32, 8, 64, 16), (8, 2, 128, 16),
-                                        (12, 1, 112, 16), (2, 1, 256, 32)])
+                                        (12, 1, 112, 16), (2, 1, 256, 32), (20, 1, 16, 8)])
 @pytest.mark.parametrize("splits", [1, 3, 7])
 @pytest.mark.parametrize("window", [0, 11])
 def test_attn_decode(dtype, H, KV, d, bs, splits, window):
@@ -366,7 +370,7 @@ def test_attn_far_key_stands_out():
     """One key among hundreds carries the weight: q and that key are scaled so that its score
     dominates; a kernel that drops or misplaces a page shows at once."""
     H, KV, d, bs = 4, 2, 64, 16
-    for far in (0, 15, 16, 255, 256, 511):
+    for far in (0, 15, 16, 255, 256, 511, 599):
         seq_lens = [600]
         paged = Paged(seq_lens, KV, d, bs, torch.float32, seed=far)
         g = torch.Generator().manual_seed(far)
@@ -390,9 +394,19 @@ def test_attn_far_key_stands_out():
                               None, 1, cu.to(DEV), ctx.to(DEV), out, H, KV, d, 1 / math.sqrt(d), 0,
                               splits, ws)
             torch.testing.assert_close(out.cpu(), want, atol=2e-5, rtol=2e-5)
+            # the same through the matrix-core kernel (operands rounded to bf16)
+            b16 = torch.bfloat16
+            outb = torch.zeros(1, H * d, dtype=b16, device=DEV)
+            ops().attn_decode(buf.to(b16).to(DEV), paged.k.to(b16).to(DEV), paged.v.to(b16).to(DEV),
+                              paged.table.to(DEV), None, 1, cu.to(DEV), ctx.to(DEV), outb, H, KV, d,
+                              1 / math.sqrt(d), 0, splits, ws)
+            wantb = plain.causal_attention(q.to(b16).float(), paged.keys[0].to(b16).float(),
+                                           paged.values[0].to(b16).float(), 1 / math.sqrt(d), 599)
+            torch.testing.assert_close(outb.float().cpu(), wantb.reshape(1, H * d), atol=2e-2, rtol=2e-2)
+            assert (outb.float().cpu().reshape(H, d)[0] - paged.values[0][far, 0]).abs().max() < 0.1
         out = torch.zeros(1, H * d, device=DEV)
         ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
-                           cu.to(DEV), ctx.to(DEV), prefill_work([1], H // KV).to(DEV), out,
+                           cu.to(DEV), ctx.to(DEV), prefill_work([1], H // KV, torch.float32, d, bs).to(DEV), out,
                            H, KV, d, 1 / math.sqrt(d), 0)
         torch.testing.assert_close(out.cpu(), want, atol=2e-5, rtol=2e-5)
 
@@ -414,7 +428,7 @@ def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
     cos_full, sin_full = plain.rope_cos_sin(torch.arange(40), inv_freq)
     cos_t, sin_t = cos_full[:, : rot // 2].contiguous(), sin_full[:, : rot // 2].contiguous()
     kp = torch.zeros(nb, KV, bs, d, dtype=dtype, device=DEV)
-    vp = torch.zeros(nb, KV, bs, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(nb, KV, d, bs, dtype=dtype, device=DEV)
     dev_qkv = qkv.to(DEV).clone()
     ops().rope_kvwrite(dev_qkv, positions.to(DEV), seq_of.to(DEV), cos_t.to(DEV), sin_t.to(DEV),
                        table.to(DEV), kp, vp, H, KV, d)
@@ -445,7 +459,7 @@ def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
         if page < 0:
             continue
         torch.testing.assert_close(kp[page, :, off], want_k[t], **tol(dtype))
-        torch.testing.assert_close(vp[page, :, off], vf[t], **tol(dtype))
+        torch.testing.assert_close(vp[page, :, :, off], vf[t], **tol(dtype))
     # nothing else was written
     written = torch.zeros(nb, bs, dtype=torch.bool)
     for t in range(n):
@@ -453,6 +467,7 @@ def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
         if int(table[s, p // bs]) >= 0:
             written[int(table[s, p // bs]), p % bs] = True
     assert (kp.abs().sum((1, 3))[~written] == 0).all()
+    assert (vp.abs().sum((1, 2))[~written] == 0).all()
 
 
 def test_sample_greedy_and_filters():

@@ -107,12 +107,13 @@ def test_embedding_and_head_parts(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bs", [4, 8])
 @pytest.mark.parametrize("H,KV,d,window", [(6, 2, 16, None), (3, 1, 48, 7), (4, 4, 32, None)])
-def test_attention_part_over_portions(dtype, H, KV, d, window):
+def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
     """The attention part alone: a sequence fed in three portions (the last a single token) beside
     a second whole sequence gives the plain whole-sequence attention block; q and k projections
     are scaled so the scores are peaked."""
-    hidden, bs = 40, 4
+    hidden = 40
     rot = RotaryPositions(d, 1000.0)
     rot.prepare(64, DEV)
     part = PagedAttention("a", hidden, H, KV, d, rot, window=window)
@@ -124,7 +125,7 @@ def test_attention_part_over_portions(dtype, H, KV, d, window):
     cache = CacheManager(bs, [CacheGroup((0,), KV, d, window)], 24)
     ls = LayerState(group=0, owns_cache=True,
                     k_pages=torch.zeros(24, KV, bs, d, dtype=dtype, device=DEV),
-                    v_pages=torch.zeros(24, KV, bs, d, dtype=dtype, device=DEV))
+                    v_pages=torch.zeros(24, KV, d, bs, dtype=dtype, device=DEV))
     xs = {"s": rand(21, hidden, seed=14).to(dtype), "t": rand(9, hidden, seed=15).to(dtype)}
     cfg = {"num_attention_heads": H, "num_key_value_heads": KV, "head_dim": d}
     want = {}
@@ -171,7 +172,7 @@ def test_pre_norm_block(dtype):
     cache = CacheManager(4, [CacheGroup((0,), KV, d, None)], 8)
     cache.allocate("r", 7)
     ls = LayerState(group=0, owns_cache=True, k_pages=torch.zeros(8, KV, 4, d, dtype=dtype, device=DEV),
-                    v_pages=torch.zeros(8, KV, 4, d, dtype=dtype, device=DEV))
+                    v_pages=torch.zeros(8, KV, d, 4, dtype=dtype, device=DEV))
     step = make_step([StepEntry("r", [0] * 7, 0, "none")], cache, dtype)
     residual = x.clone().to(DEV)
     block.forward(residual, step, ls)
