@@ -140,19 +140,22 @@ constexpr int depth(int mt, int nt, int at) {
   return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : (mt * nt == 1 ? 8 : mt * nt <= 4 ? 4 : 2);
 }
 
-template <int MT, int NT, int AT, int EPI>
+// RW: rows of W one workgroup owns (16, 8 or 4).  With fewer than 16 the instruction's other
+// rows repeat them (same addresses, no extra memory traffic) and are dropped at the store: it
+// trades matrix-core work, which is free here, for more workgroups when N is small.
+template <int MT, int NT, int AT, int EPI, int RW>
 __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
     int K, int lda, int ldc, int m_base, float eps, RopeEpi rp) {
   extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
   const int nw = blockDim.x / KVF_WAVE;
-  const int n0 = blockIdx.x * 16 * NT;
+  const int n0 = blockIdx.x * RW * NT;
   const int r16 = lane % 16, kg = lane / 16;
   const bf16_t* wp[NT];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    int wrow = n0 + j * 16 + r16;
+    int wrow = n0 + j * RW + r16 % RW;
     if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
     wp[j] = W + static_cast<size_t>(wrow) * K + kg * 8;
   }
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     int arow = m_base + t * 16 + r16;
-    if (arow >= M) arow = M - 1;
+    if (arow >= M) arow = M - 1;  // rows past M repeat the last one and are never stored
     aoff[t] = static_cast<size_t>(arow) * lda + kg * 8;
   }
   const bf16_t* Ab = static_cast<const bf16_t*>(Av);
@@ -236,8 +239,8 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       for (int w = 0; w < nw; ++w)
         s += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * KVF_WAVE + l) * 4);
       const int m = m_base + t * 16 + l % 16;
-      const int n = n0 + j * 16 + 4 * (l / 16);
-      if (m >= M || n >= N) continue;
+      const int n = n0 + j * RW + 4 * (l / 16);
+      if (m >= M || n >= N || 4 * (l / 16) >= RW) continue;
       if (AT) {
         float tot = 0.f;
         for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
@@ -249,27 +252,29 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 }
 
 int g_waves_override = 0;
+int g_rows_override = 0;
 
-// Waves per workgroup: enough workgroups x waves to keep every CU streaming (about 2048 waves
-// in all), at least one k-step per wave.
+// Waves per workgroup, as measured on the shapes of a 1B-parameter decoder: eight when the grid
+// is small (fewer leave loads unhidden, sixteen crowd the CU), four when a thousand or more
+// workgroups already fill every CU several times; at least one k-step per wave.
 int pick_waves(int groups, int K) {
   const int ksteps = (K + 31) / 32;
-  int nw = g_waves_override > 0 ? g_waves_override : (2048 + groups - 1) / groups;
+  int nw = g_waves_override > 0 ? g_waves_override : (groups >= 1024 ? 4 : 8);
   if (nw > 16) nw = 16;
   if (nw > ksteps) nw = ksteps;
   if (nw < 1) nw = 1;
   return nw;
 }
 
-template <int MT, int NT, int AT, int EPI>
+template <int MT, int NT, int AT, int EPI, int RW = 16>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
                int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
-  const int groups = (N + 16 * NT - 1) / (16 * NT);
+  const int groups = (N + RW * NT - 1) / (RW * NT);
   int nw = pick_waves(groups, K);
   if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
   const dim3 grid(groups), block(nw * KVF_WAVE);
   const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, RW>), grid, block, lds, s, A, W, C, M, N, K,
                      lda, ldc, m_base, eps, rp);
   return kvf_last_error();
 }
@@ -285,6 +290,11 @@ int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int 
       return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
     if (tiles >= 512)
       return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+  }
+  if (MT == 1) {
+    const int rw = g_rows_override > 0 ? g_rows_override : 16;  // fewer rows measured no gain
+    if (rw == 4) return launch_one<1, 1, AT, EPI, 4>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (rw == 8) return launch_one<1, 1, AT, EPI, 8>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
   }
   return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
 }
@@ -317,8 +327,10 @@ int launch_epi(const void* A, const bf16_t* W, void* C, int epi, int M, int N, i
 }
 }  // namespace
 
-// For measurements: force the number of waves per workgroup (0 = choose by shape).
+// For measurements: force the number of waves per workgroup and the rows of W per workgroup
+// (0 = choose by shape).
 KVF_EXPORT void kvf_gemm_bf16_set_waves(int waves) { g_waves_override = waves; }
+KVF_EXPORT void kvf_gemm_bf16_set_rows(int rows) { g_rows_override = rows; }
 
 // a_type: 0 = bf16 rows, 1 = fp32 rows normalised by rsqrt(mean(x^2) + eps) in the kernel.
 // epi: 0 store fp32, 1 store bf16, 2 add into fp32, 3 SwiGLU pairs -> bf16 [M, N/2].

@@ -56,7 +56,25 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
   if (!(temp > 0.f)) {  // greedy
     float best = -INFINITY;
     int bi = V;
-    for (int i = tid; i < V; i += THREADS) {
+    // rows of 4 floats at a time where the row is 16-byte aligned; several loads in flight
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    const int v4 = vec ? V / 4 : 0;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    for (int i0 = tid; i0 < v4; i0 += 4 * THREADS) {
+      float4 r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        r[u] = i0 + u * THREADS < v4 ? x4[i0 + u * THREADS] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int base = 4 * (i0 + u * THREADS);
+        const float e[4] = {r[u].x, r[u].y, r[u].z, r[u].w};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (e[c] > best || (e[c] == best && base + c < bi)) { best = e[c]; bi = base + c; }
+      }
+    }
+    for (int i = 4 * v4 + tid; i < V; i += THREADS) {
       const float v = x[i];
       if (v > best || (v == best && i < bi)) { best = v; bi = i; }
     }

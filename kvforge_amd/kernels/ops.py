@@ -162,8 +162,11 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 
 
 # ------------------------------------------------------------------------------ matrix products
-# Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.
-SKINNY_MAX_M = 128
+# Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16: one
+# 16-row tile.  With more rows the library's bf16 product measured faster on every shape of a
+# 1B-parameter decoder (it splits K across workgroups), and the reference's engine uses a
+# library product there as well.
+SKINNY_MAX_M = 16
 FUSED_NORM_MAX_M = 16
 _GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
 
@@ -212,14 +215,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if not accumulate:
         _tcode(out.dtype)
     if a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0:
-        if m <= SKINNY_MAX_M or out_kind == 0:
+        if m <= SKINNY_MAX_M:
             f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
             _ok(f(a.data_ptr(), 0, w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
                   _stream()), "gemm_bf16")
         elif accumulate:
-            # many rows: the library's bf16 product (as the reference's engine uses one), then
-            # the residual sum in fp32
+            # many rows: the library's bf16 product, then the residual sum in fp32
             out.add_(torch.mm(a, w.t()))
+        elif out.dtype == F32:
+            out.copy_(torch.mm(a, w.t()))
         else:
             torch.mm(a, w.t(), out=out)
         return
@@ -301,12 +305,14 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
           _stream()), "gemm_qkv_rope")
 
 
-def set_gemm_waves(waves: int) -> None:
-    """Measurement aid: force the waves per workgroup of the MFMA kernel (0 = by shape)."""
+def set_gemm_waves(waves: int, rows: int = 0) -> None:
+    """Measurement aid: force the waves per workgroup and the rows of W per workgroup of the
+    MFMA kernel (0 = by shape)."""
     lib = library.load("gemm_bf16")
-    lib.kvf_gemm_bf16_set_waves.argtypes = [c_int]
-    lib.kvf_gemm_bf16_set_waves.restype = None
-    lib.kvf_gemm_bf16_set_waves(int(waves))
+    for fn, v in ((lib.kvf_gemm_bf16_set_waves, waves), (lib.kvf_gemm_bf16_set_rows, rows)):
+        fn.argtypes = [c_int]
+        fn.restype = None
+        fn(int(v))
 
 
 # ------------------------------------------------------------------------------ attention

