@@ -1,6 +1,7 @@
 // Paged causal attention for bf16 on the matrix cores, for query runs (prefill) and for single
-// tokens (decode).  No tile of K or V passes through LDS: every operand fragment is loaded
-// from the pages straight into the registers layout the instruction wants.
+// tokens (decode).  Every operand fragment is loaded from the pages in the register layout the
+// instruction wants (no transposes); for query runs the four waves of a workgroup share the
+// fragments of a key block through LDS, each loading a quarter of them one block ahead.
 //
 // Rows: row r of a (sequence, kv head) is (query token r / G, head r % G of the group), so the
 // G query heads that share a kv head share every K/V fragment.  A wave owns tiles of 16 rows;
@@ -18,33 +19,62 @@
 //   operand by a rounding to bf16 alone; softmax itself is fp32.
 // Key j is visible to a query at position p iff j <= p, j < context length and, with a window
 // w > 0, j > p - w.  Scores are scaled after the dot product.
+// The softmax reference of a row (what is subtracted before exp) is raised only when some score
+// of the wave exceeds it by more than LAZY (in log2 units): exp(s - ref) then stays below
+// 2^LAZY, sums and accumulators need no rescaling in most blocks, and the result is the same
+// softmax (any reference cancels in the final division).
 //
-// SPLIT = false (runs): a workgroup takes 4 * RT consecutive row tiles of one (sequence, kv
-//   head) from a work list; its waves are independent.
-// SPLIT = true (few rows, long key range): a workgroup takes one row tile and one of `splits`
-//   cuts of the key range; its four waves take the blocks of that cut in turn and are merged
-//   through LDS; with splits > 1 partial (max, sum, accumulator) go to a workspace that
+// Loads are never predicated: a lane without a valid page reads page 0 and its fragment is
+// cleared by a mask when it is consumed, so nothing waits on a load before its data is needed.
+//
+// Query runs: a workgroup takes 4 * RT consecutive row tiles of one (sequence, kv head) from a
+//   work list.  Three stages are in flight: page lookups two blocks ahead, fragment loads one
+//   block ahead (registers, then the other half of a double LDS buffer), products of this block.
+// Few rows, long key range: a workgroup takes one row tile and one of `splits` cuts of the key
+//   range; its four waves take the blocks of that cut in turn and are merged through LDS; with
+//   splits > 1 partial (max, sum, accumulator) go to a workspace that
 //   `attn_split_combine_kernel` merges in split order.
-// block_size must be a multiple of 8 (a lane's eight keys lie in one page), d a multiple of 16.
+// block_size must be a multiple of 8 (a lane's eight keys lie in one page), d a multiple of 16;
+// kernels are instantiated for each d / 16 so that no loop bound is left to run time.
 #include "common.h"
 
 namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) float f32x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int WAVES = 4;
+constexpr float LAZY = 8.f;                    // log2 headroom before a row's reference is raised
+constexpr float LOG2E = 1.4426950408889634f;
+
+// With at least two waves per SIMD asked for, a wave has at most 256 registers and the compiler
+// keeps accumulators in ordinary vector registers, where the softmax rescale can reach them
+// without copies from and to the accumulation registers in every block.
+#define KVF_VGPR_FORM(FITS) __attribute__((amdgpu_waves_per_eu((FITS) ? 2 : 1)))
 
 struct MArgs {
   int H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits;
   float scale;
+  unsigned bs_magic;  // floor(2^32 / bs) + 1: key / bs == mulhi(key, bs_magic) while key * bs < 2^32
 };
 
-__device__ __forceinline__ bf16x8 ld_frag(const bf16_t* p, bool ok) {
-  uint4 r = make_uint4(0u, 0u, 0u, 0u);
-  if (ok) r = *reinterpret_cast<const uint4*>(p);
-  return __builtin_bit_cast(bf16x8, r);
+// Position of a key in its page table: (page table entry, slot in the page)
+__device__ __forceinline__ int block_of(const MArgs& a, int key) {
+  return static_cast<int>(__umulhi(static_cast<unsigned>(key), a.bs_magic));
 }
 
-// max over the four lanes of a row (lanes j, j+16, j+32, j+48)
+__device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ bf16x8 as_frag(const uint4& r) { return __builtin_bit_cast(bf16x8, r); }
+
+// Keeps the first `live` (0..8) bf16 of a fragment, clears the rest.
+__device__ __forceinline__ uint4 keep_first(const uint4& r, int live) {
+  if (!__any(live < 8)) return r;  // nearly every fragment is whole in every lane
+  uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] &= 2 * e + 1 < live ? 0xffffffffu : (2 * e < live ? 0xffffu : 0u);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// max / sum over the four lanes of a row (lanes j, j+16, j+32, j+48)
 __device__ __forceinline__ float row_max(float v) {
   v = fmaxf(v, __shfl_xor(v, 16, KVF_WAVE));
   return fmaxf(v, __shfl_xor(v, 32, KVF_WAVE));
@@ -54,227 +84,463 @@ __device__ __forceinline__ float row_sum(float v) {
   return v + __shfl_xor(v, 32, KVF_WAVE);
 }
 
-template <int DTMAX, int RT, bool SPLIT>
-__global__ __launch_bounds__(256) void attn_mfma_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
-    const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
-    const int* __restrict__ items, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
-    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, MArgs a) {
-  constexpr int DCMAX = DTMAX / 2;  // 32-wide steps of the q.k contraction
-  extern __shared__ float lds[];    // SPLIT only: [WAVES][dt][64][4] accumulators, [WAVES][16][2]
+// What a lane needs to find its operand fragments of the key block at kb.
+struct Pages {
+  const bf16_t* k_pages;
+  const bf16_t* vt_pages;
+  const int* table;
+  int kvh, ctx, j16, kg;
+};
 
-  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
-  const int j16 = lane % 16, kg = lane / 16;
-  const int G = a.H / a.KV, D = a.d;
-  const int dt_n = D / 16, dc_n = (D + 31) / 32;
+// A page lookup: the table entry as loaded, and whether the key it was asked for exists.  The
+// two are only combined where the page is used, so that nothing waits for the load before then;
+// the lookup is issued one block before the fragment loads that need it.
+struct PageRef {
+  int page;
+  bool asked;
+  __device__ __forceinline__ bool ok(int nb) const { return asked && page >= 0 && page < nb; }
+};
+__device__ __forceinline__ PageRef page_of_key(const Pages& pg, const MArgs& a, int key) {
+  const int blk = block_of(a, key);
+  PageRef r;
+  r.page = pg.table[min(blk, a.table_stride - 1)];  // always a valid address
+  r.asked = key < pg.ctx && blk < a.table_stride;
+  return r;
+}
+// Page that holds the keys of K tile t for this lane (row i = j16 is key kb + 8*(i/4) + 4*t + i%4)
+__device__ __forceinline__ PageRef k_page(const Pages& pg, const MArgs& a, int kb, int t) {
+  return page_of_key(pg, a, kb + 8 * (pg.j16 >> 2) + 4 * t + (pg.j16 & 3));
+}
+// Page of the keys kb + 8*kg + 0..7 (one page: the page size is a multiple of 8)
+__device__ __forceinline__ PageRef v_page(const Pages& pg, const MArgs& a, int kb) {
+  return page_of_key(pg, a, kb + 8 * pg.kg);
+}
 
-  int seq, kvh, first_tile, item_index;
-  if (SPLIT) {
-    const int chunks = (G + 15) / 16;
-    item_index = blockIdx.x;
-    seq = items ? items[blockIdx.x] : static_cast<int>(blockIdx.x);
-    kvh = blockIdx.y / chunks;
-    first_tile = blockIdx.y - kvh * chunks;
-  } else {
-    item_index = 0;
-    seq = items[2 * blockIdx.x];
-    kvh = blockIdx.y;
-    first_tile = (items[2 * blockIdx.x + 1] * WAVES + wave) * RT;
+// K fragment of tile t, contraction step c, and how many of its eight elements count: none
+// without a page or where the step reaches past d (head sizes that are odd multiples of 16).
+// Offsets into the pages are counted in fragments of 16 bytes and fit 32 bits (the host checks).
+template <int DT>
+__device__ __forceinline__ uint4 k_fragment(const Pages& pg, const MArgs& a, int kb, int t, int c,
+                                            const PageRef& ref, int& live) {
+  const int key = kb + 8 * (pg.j16 >> 2) + 4 * t + (pg.j16 & 3);
+  const int slot = key - block_of(a, key) * a.bs;
+  const bool over = (DT % 2) && c == DT / 2 && pg.kg >= 2;
+  const bool ok = ref.ok(a.nb) && !over;
+  live = ok ? 8 : 0;
+  const unsigned row = (static_cast<unsigned>(ok ? ref.page : 0) * a.KV + pg.kvh) * a.bs + slot;
+  const unsigned off = row * (a.d / 8) + (over ? 0 : c * 4 + pg.kg);
+  return ld16(pg.k_pages + static_cast<size_t>(off) * 8);
+}
+// V^T fragment of element tile dt (row i = j16 is element dt*16 + i), slots are keys
+// kb + 8*kg + 0..7.  Keys at or past the context length hold whatever an earlier owner of the
+// page left there: they do not count.
+__device__ __forceinline__ uint4 v_fragment(const Pages& pg, const MArgs& a, int kb, int dt,
+                                            const PageRef& ref, int& live) {
+  const int key = kb + 8 * pg.kg;
+  const int slot = key - block_of(a, key) * a.bs;
+  const bool ok = ref.ok(a.nb);
+  live = ok ? min(pg.ctx - key, 8) : 0;
+  const unsigned row = (static_cast<unsigned>(ok ? ref.page : 0) * a.KV + pg.kvh) * a.d + dt * 16 + pg.j16;
+  const unsigned off = row * (a.bs / 8) + slot / 8;
+  return ld16(pg.vt_pages + static_cast<size_t>(off) * 8);
+}
+
+// The rows a lane works for: one per row tile.
+template <int RT> struct Rows {
+  bool ok[RT];
+  int tok[RT], head[RT];
+  int first[RT];       // first visible key of the row
+  unsigned span[RT];   // visible keys are first .. first + span; a row that is none has first < 0
+};
+
+// One key block for the row tiles of a wave: scores, lazy softmax update, P * V.
+// References live in log2 units: scale2 = scale * log2(e) > 0 is applied inside the exponent.
+template <int DT, int RT>
+__device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2], const bf16x8 (&vf)[DT],
+                                             const bf16x8 (&qf)[RT][(DT + 1) / 2], const Rows<RT>& rows,
+                                             int kb, int kg, bool edge, float scale2, float (&m_ref)[RT], float (&l_run)[RT],
+                                             f32x4 (&acc)[RT][DT]) {
+  constexpr int DC = (DT + 1) / 2;
+  f32x4 s[RT][2];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DC; ++c)
+        s[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][c], qf[rt][c], s[rt][t], 0, 0, 0);
+    }
+  // lane holds keys kb + 8*kg + 4*t + r of its row
+  if (edge) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = kb + 8 * kg + 4 * t + r;
+          const bool vis = static_cast<unsigned>(key - rows.first[rt]) <= rows.span[rt];
+          s[rt][t][r] = vis ? s[rt][t][r] : -INFINITY;
+        }
   }
-  if (seq < 0 || seq >= a.n_seqs) return;
-  const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
-  const int start = ctx - qlen;
-  const int rows_total = qlen * G;
-  const int* table = block_table + static_cast<size_t>(seq) * a.table_stride;
-  const bool seq_ok = qlen > 0 && start >= 0;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    // the scale is positive: the largest raw score is the largest scaled one
+    const float bm = scale2 * fmaxf(fmaxf(fmaxf(s[rt][0][0], s[rt][0][1]), fmaxf(s[rt][0][2], s[rt][0][3])),
+                                    fmaxf(fmaxf(s[rt][1][0], s[rt][1][1]), fmaxf(s[rt][1][2], s[rt][1][3])));
+    if (__any(bm > m_ref[rt] + LAZY)) {
+      const float m_new = fmaxf(m_ref[rt], row_max(bm));
+      if (m_new != m_ref[rt]) {
+        const float corr = __builtin_amdgcn_exp2f(m_ref[rt] - m_new);  // 0 from a reference of -inf
+        l_run[rt] *= corr;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc[rt][t] *= corr;
+        m_ref[rt] = m_new;
+      }
+    }
+    // a row that has seen no key yet has only -inf scores: any finite reference gives zeros
+    const float m_use = m_ref[rt] == -INFINITY ? 0.f : m_ref[rt];
+    f32x8 p;
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float e = __builtin_amdgcn_exp2f(fmaf(s[rt][t][r], scale2, -m_use));
+        p[4 * t + r] = e;
+        psum += e;
+      }
+    l_run[rt] += psum;  // this lane's share of the row's sum
+    const bf16x8 pf = __builtin_convertvector(p, bf16x8);
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+      acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t], pf, acc[rt][t], 0, 0, 0);
+  }
+}
 
-  // ---- this lane's rows and their query fragments
-  bool row_ok[RT];
-  int row_pos[RT], row_tok[RT], row_head[RT];
-  bf16x8 qf[RT][DCMAX];
-  int pos_min = 0x7fffffff, pos_max = -1;
+__device__ __forceinline__ uint2 pack4(const f32x4& v, float f) {
+  uint2 pk;
+  pk.x = static_cast<uint32_t>(f32_to_bf16(v[0] * f)) | (static_cast<uint32_t>(f32_to_bf16(v[1] * f)) << 16);
+  pk.y = static_cast<uint32_t>(f32_to_bf16(v[2] * f)) | (static_cast<uint32_t>(f32_to_bf16(v[3] * f)) << 16);
+  return pk;
+}
+
+// Sets up the rows of `RT` tiles starting at `first_tile`; returns the positions they span.
+template <int DT, int RT>
+__device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int q0, int qlen, int start,
+                                           int kvh, int first_tile, int j16, int kg, bool seq_ok,
+                                           Rows<RT>& rows, bf16x8 (&qf)[RT][(DT + 1) / 2], int& pos_min,
+                                           int& pos_max) {
+  const int G = a.H / a.KV, D = a.d, rows_total = qlen * G;
+  pos_min = 0x7fffffff;
+  pos_max = -1;
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     const int row = (first_tile + rt) * 16 + j16;
-    row_ok[rt] = seq_ok && row < rows_total;
-    const int tok = row_ok[rt] ? row / G : 0;
-    row_tok[rt] = tok;
-    row_head[rt] = kvh * G + (row_ok[rt] ? row - tok * G : 0);
-    row_pos[rt] = start + tok;
-    const int t_lo = (first_tile + rt) * 16 / G;                       // first token of the tile
-    int t_hi = ((first_tile + rt) * 16 + 15) / G;                      // last token of the tile
-    if (t_hi > qlen - 1) t_hi = qlen - 1;
+    rows.ok[rt] = seq_ok && row < rows_total;
+    const int tok = rows.ok[rt] ? row / G : 0;
+    rows.tok[rt] = tok;
+    rows.head[rt] = kvh * G + (rows.ok[rt] ? row - tok * G : 0);
+    {  // the row's position is below the context length, so it is its last visible key
+      const int pos = start + tok;
+      const int first = a.window > 0 && pos - a.window + 1 > 0 ? pos - a.window + 1 : 0;
+      rows.first[rt] = rows.ok[rt] ? first : -1;
+      rows.span[rt] = rows.ok[rt] ? static_cast<unsigned>(pos - first) : 0u;
+    }
     if (seq_ok && (first_tile + rt) * 16 < rows_total) {
-      pos_min = min(pos_min, start + t_lo);
+      int t_hi = ((first_tile + rt) * 16 + 15) / G;
+      if (t_hi > qlen - 1) t_hi = qlen - 1;
+      pos_min = min(pos_min, start + (first_tile + rt) * 16 / G);
       pos_max = max(pos_max, start + t_hi);
     }
-    const bf16_t* qp = q + static_cast<size_t>(q0 + tok) * a.q_stride + row_head[rt] * D + kg * 8;
+    const bf16_t* qp = q + static_cast<size_t>(q0 + tok) * a.q_stride + rows.head[rt] * D + kg * 8;
 #pragma unroll
-    for (int c = 0; c < DCMAX; ++c)
-      qf[rt][c] = ld_frag(qp + c * 32, row_ok[rt] && c < dc_n && c * 32 + kg * 8 < D);
+    for (int c = 0; c < (DT + 1) / 2; ++c) {
+      const bool ok = rows.ok[rt] && c * 32 + kg * 8 < D;
+      qf[rt][c] = as_frag(ok ? ld16(qp + c * 32) : make_uint4(0u, 0u, 0u, 0u));
+    }
   }
-  // ---- key range of this wave
+}
+
+// ------------------------------------------------------------------------------------ query runs
+// SHARE: the waves stage the fragments of each key block in LDS for each other; otherwise every
+// wave loads all of them itself.
+template <int DT, int RT, bool SHARE>
+__global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
+    const int* __restrict__ work, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    bf16_t* __restrict__ out, MArgs a) {
+  constexpr int DC = (DT + 1) / 2;
+  constexpr int N_K = 2 * DC, N_FRAG = N_K + DT;          // fragments of a key block
+  constexpr int FPW = (N_FRAG + WAVES - 1) / WAVES;       // fragments a wave stages per block
+  extern __shared__ uint4 frag_lds[];                     // SHARE: [2][N_FRAG][64]
+
+  const int lane = threadIdx.x % KVF_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KVF_WAVE);  // the same in all lanes
+  const int j16 = lane % 16, kg = lane / 16;
+  const int G = a.H / a.KV, D = a.d;
+  // The kv heads of the upper half of the grid walk the work list backwards: where two
+  // workgroups half a grid apart land on one compute unit, a long run of keys meets a short one.
+  const int wi = blockIdx.y >= (gridDim.y + 1) / 2 ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+  const int seq = work[2 * wi], kvh = blockIdx.y;
+  if (seq < 0 || seq >= a.n_seqs) return;
+  const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
+  const int start = ctx - qlen;
+  const bool seq_ok = qlen > 0 && start >= 0;
+  const int wg_tile = work[2 * wi + 1] * WAVES * RT;
+  const Pages pg{k_pages, vt_pages, block_table + static_cast<size_t>(seq) * a.table_stride, kvh, ctx,
+                 j16, kg};
+
+  Rows<RT> rows;
+  bf16x8 qf[RT][DC];
+  int pos_min, pos_max;
+  setup_rows<DT, RT>(q, a, q0, qlen, start, kvh, wg_tile + wave * RT, j16, kg, seq_ok, rows, qf, pos_min,
+                     pos_max);
+  // key range of this wave, and of the workgroup (tiles wg_tile .. wg_tile + 4*RT - 1)
+  int lo_w = 0, hi_w = -1;
+  if (pos_max >= 0) {
+    hi_w = pos_max < ctx - 1 ? pos_max : ctx - 1;
+    if (a.window > 0 && pos_min - a.window + 1 > 0) lo_w = pos_min - a.window + 1;
+  }
+  int lo_g = 0, hi_g = -1;
+  if (seq_ok && wg_tile * 16 < qlen * G) {
+    int t_hi = ((wg_tile + WAVES * RT) * 16 - 1) / G;
+    if (t_hi > qlen - 1) t_hi = qlen - 1;
+    hi_g = start + t_hi < ctx - 1 ? start + t_hi : ctx - 1;
+    const int p_lo = start + wg_tile * 16 / G;
+    if (a.window > 0 && p_lo - a.window + 1 > 0) lo_g = p_lo - a.window + 1;
+  }
+  const float scale2 = a.scale * LOG2E;
+
+  float m_ref[RT], l_run[RT];
+  f32x4 acc[RT][DT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    m_ref[rt] = -INFINITY;
+    l_run[rt] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (SHARE) {
+    // fragment f of a block: K (tile f / DC, step f % DC) for f < N_K, then V^T element tiles;
+    // wave w stages fragments w, w + 4, ...
+    const int kb_first = (lo_g / 32) * 32;
+    uint4 stage[FPW];
+    PageRef page[FPW];
+    int live[FPW];
+    auto locate = [&](int kb) {
+#pragma unroll
+      for (int i = 0; i < FPW; ++i) {
+        const int f = wave + i * WAVES;
+        page[i] = f < N_K ? k_page(pg, a, kb, f / DC) : v_page(pg, a, kb);
+      }
+    };
+    auto fetch = [&](int kb) {
+#pragma unroll
+      for (int i = 0; i < FPW; ++i) {
+        const int f = wave + i * WAVES;
+        if (f < N_K) stage[i] = k_fragment<DT>(pg, a, kb, f / DC, f % DC, page[i], live[i]);
+        else if (f < N_FRAG) stage[i] = v_fragment(pg, a, kb, f - N_K, page[i], live[i]);
+      }
+    };
+    auto put = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < FPW; ++i) {
+        const int f = wave + i * WAVES;
+        if (f < N_FRAG) frag_lds[(buf * N_FRAG + f) * KVF_WAVE + lane] = keep_first(stage[i], live[i]);
+      }
+    };
+    if (kb_first <= hi_g) {
+      locate(kb_first);
+      fetch(kb_first);
+      locate(kb_first + 32);
+      put(0);
+    }
+    // Everything loaded so far (the query fragments among it) has to be there before the loop:
+    // otherwise the compiler, not knowing how many loads a first pass through the loop still has
+    // ahead of them, waits for all loads before the first product of every pass.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    int buf = 0;
+    for (int kb = kb_first; kb <= hi_g; kb += 32) {
+      const bool more = kb + 32 <= hi_g;
+      if (more) {
+        fetch(kb + 32);   // its pages were looked up a block ago
+        locate(kb + 64);  // nothing past the context is looked up
+      }
+      if (kb <= hi_w && kb + 31 >= lo_w) {
+        bf16x8 kf[2][DC], vf[DT];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int c = 0; c < DC; ++c)
+            kf[t][c] = as_frag(frag_lds[(buf * N_FRAG + t * DC + c) * KVF_WAVE + lane]);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) vf[t] = as_frag(frag_lds[(buf * N_FRAG + N_K + t) * KVF_WAVE + lane]);
+        const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
+        block_update<DT, RT>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+      }
+      if (more) put(buf ^ 1);
+      __syncthreads();
+      buf ^= 1;
+    }
+  } else {
+    PageRef pk[2] = {k_page(pg, a, (lo_w / 32) * 32, 0), k_page(pg, a, (lo_w / 32) * 32, 1)};
+    PageRef pv = v_page(pg, a, (lo_w / 32) * 32);
+    for (int kb = (lo_w / 32) * 32; kb <= hi_w; kb += 32) {
+      uint4 kr[2][DC], vr[DT];
+      int kl[2][DC], vl;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int c = 0; c < DC; ++c) kr[t][c] = k_fragment<DT>(pg, a, kb, t, c, pk[t], kl[t][c]);
+#pragma unroll
+      for (int t = 0; t < DT; ++t) vr[t] = v_fragment(pg, a, kb, t, pv, vl);
+      pk[0] = k_page(pg, a, kb + 32, 0);
+      pk[1] = k_page(pg, a, kb + 32, 1);
+      pv = v_page(pg, a, kb + 32);
+      bf16x8 kf[2][DC], vf[DT];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int c = 0; c < DC; ++c) kf[t][c] = as_frag(keep_first(kr[t][c], kl[t][c]));
+#pragma unroll
+      for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(vr[t], vl));
+      const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
+      block_update<DT, RT>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+    }
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const float l = row_sum(l_run[rt]);
+    if (!rows.ok[rt]) continue;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t* o = out + static_cast<size_t>(q0 + rows.tok[rt]) * a.o_stride + rows.head[rt] * D + 4 * kg;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) *reinterpret_cast<uint2*>(o + t * 16) = pack4(acc[rt][t], inv);
+  }
+}
+
+// ------------------------------------------------------------------------- few rows, split keys
+// TWO: a wave holds the fragments of two blocks, loading one while it consumes the other.
+template <int DT, bool TWO>
+__global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
+    const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, MArgs a) {
+  constexpr int DC = (DT + 1) / 2;
+  extern __shared__ float lds[];  // [WAVES][DT][64][4] accumulators, then [WAVES][16][2]
+
+  const int lane = threadIdx.x % KVF_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KVF_WAVE);  // the same in all lanes
+  const int j16 = lane % 16, kg = lane / 16;
+  const int G = a.H / a.KV, D = a.d;
+  const int chunks = (G + 15) / 16;
+  const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
+  if (seq < 0 || seq >= a.n_seqs) return;
+  const int kvh = blockIdx.y / chunks, tile = blockIdx.y - kvh * chunks;
+  const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
+  const int start = ctx - qlen;
+  const bool seq_ok = qlen > 0 && start >= 0;
+  const Pages pg{k_pages, vt_pages, block_table + static_cast<size_t>(seq) * a.table_stride, kvh, ctx,
+                 j16, kg};
+  Rows<1> rows;
+  bf16x8 qf[1][DC];
+  int pos_min, pos_max;
+  setup_rows<DT, 1>(q, a, q0, qlen, start, kvh, tile, j16, kg, seq_ok, rows, qf, pos_min, pos_max);
   int lo = 0, hi = -1;
   if (pos_max >= 0) {
     hi = pos_max < ctx - 1 ? pos_max : ctx - 1;
     if (a.window > 0 && pos_min - a.window + 1 > 0) lo = pos_min - a.window + 1;
   }
-  int kb_begin = (lo / 32) * 32, kb_step = 32, kb_end = hi + 1;
-  if (SPLIT) {
-    const int blocks = hi >= kb_begin ? (hi - kb_begin) / 32 + 1 : 0;
-    int per = (blocks + a.splits - 1) / a.splits;
-    per = (per + WAVES - 1) / WAVES * WAVES;          // whole rounds of the four waves
-    const int b0 = blockIdx.z * per;
-    kb_end = min(kb_end, kb_begin + (b0 + per) * 32);
-    kb_begin += (b0 + wave) * 32;
-    kb_step = 32 * WAVES;
-  }
+  const int kb0 = (lo / 32) * 32;
+  const int blocks = hi >= kb0 ? (hi - kb0) / 32 + 1 : 0;
+  int per = (blocks + a.splits - 1) / a.splits;
+  per = (per + WAVES - 1) / WAVES * WAVES;  // whole rounds of the four waves
+  const int kb_end = min(hi + 1, kb0 + (static_cast<int>(blockIdx.z) + 1) * per * 32);
+  const int kb_begin = kb0 + (blockIdx.z * per + wave) * 32;
+  constexpr int STEP = 32 * WAVES;
+  const float scale2 = a.scale * LOG2E;
 
-  float m_run[RT], l_run[RT];
-  f32x4 acc[RT][DTMAX];
+  float m_ref[1] = {-INFINITY}, l_run[1] = {0.f};
+  f32x4 acc[1][DT];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    m_run[rt] = -INFINITY;
-    l_run[rt] = 0.f;
-#pragma unroll
-    for (int t = 0; t < DTMAX; ++t) acc[rt][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int t = 0; t < DT; ++t) acc[0][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int kb = kb_begin; kb < kb_end; kb += kb_step) {
-    // ---- K fragments: tile t, row i = j16 is key kb + 8*(i/4) + 4*t + i%4
-    bf16x8 kf[2][DCMAX];
+  // The register buffers are named apart (an index chosen at run time would put them in
+  // scratch); the pages of a block are looked up one block before its fragments are loaded.
+  struct Raw {
+    uint4 k[2][DC], v[DT];
+    int kl[2][DC], vl;
+  };
+  Raw A, B;
+  PageRef pA[3], pB[3];
+  auto locate = [&](int kb, PageRef (&p)[3]) {
+    p[0] = k_page(pg, a, kb, 0);
+    p[1] = k_page(pg, a, kb, 1);
+    p[2] = v_page(pg, a, kb);
+  };
+  auto fetch = [&](int kb, const PageRef (&p)[3], Raw& r) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int key = kb + 8 * (j16 >> 2) + 4 * t + (j16 & 3);
-      const int blk = key / a.bs;
-      int page = -1;
-      if (key < ctx && blk < a.table_stride) page = table[blk];
-      const bool ok = page >= 0 && page < a.nb;
-      const bf16_t* kp = k_pages + ((static_cast<size_t>(ok ? page : 0) * a.KV + kvh) * a.bs +
-                                    (key - blk * a.bs)) * D + kg * 8;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int c = 0; c < DCMAX; ++c)
-        kf[t][c] = ld_frag(kp + c * 32, ok && c < dc_n && c * 32 + kg * 8 < D);
-    }
-    // ---- V^T fragments: row i = j16 is element dt*16 + i, slots are keys kb + 8*kg + 0..7
-    bf16x8 vf[DTMAX];
-    {
-      const int key = kb + 8 * kg;
-      const int blk = key / a.bs;
-      int page = -1;
-      if (key < ctx && blk < a.table_stride) page = table[blk];
-      const bool ok = page >= 0 && page < a.nb;
-      const bf16_t* vp = vt_pages + ((static_cast<size_t>(ok ? page : 0) * a.KV + kvh) * D + j16) * a.bs +
-                         (key - blk * a.bs);
-      // keys at or past the context length hold whatever an earlier owner left: clear them
-      const int live = ctx - key;  // > 0 when ok
+      for (int c = 0; c < DC; ++c) r.k[t][c] = k_fragment<DT>(pg, a, kb, t, c, p[t], r.kl[t][c]);
 #pragma unroll
-      for (int t = 0; t < DTMAX; ++t) {
-        vf[t] = ld_frag(vp + static_cast<size_t>(t) * 16 * a.bs, ok && t < dt_n);
-        if (ok && live < 8) {
-          uint4 r = __builtin_bit_cast(uint4, vf[t]);
-          uint32_t w[4] = {r.x, r.y, r.z, r.w};
+    for (int t = 0; t < DT; ++t) r.v[t] = v_fragment(pg, a, kb, t, p[2], r.vl);
+  };
+  auto consume = [&](int kb, const Raw& r) {
+    bf16x8 kf[2][DC], vf[DT];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (2 * e >= live) w[e] = 0u;
-            else if (2 * e + 1 >= live) w[e] &= 0xffffu;
-          }
-          vf[t] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
-        }
-      }
-    }
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int c = 0; c < DC; ++c) kf[t][c] = as_frag(keep_first(r.k[t][c], r.kl[t][c]));
+#pragma unroll
+    for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(r.v[t], r.vl));
     const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      f32x4 s[2];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int c = 0; c < DCMAX; ++c)
-          if (c < dc_n) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][c], qf[rt][c], s[t], 0, 0, 0);
+    block_update<DT, 1>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+  };
+  // the query fragments have to be there before the loops (see the note in the runs kernel)
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  if (TWO) {
+    if (kb_begin < kb_end) {
+      locate(kb_begin, pA);
+      locate(kb_begin + STEP, pB);
+      fetch(kb_begin, pA, A);
+    }
+    for (int kb = kb_begin; kb < kb_end; kb += 2 * STEP) {
+      const bool second = kb + STEP < kb_end;
+      if (second) fetch(kb + STEP, pB, B);
+      locate(kb + 2 * STEP, pA);
+      consume(kb, A);
+      if (second) {
+        if (kb + 2 * STEP < kb_end) fetch(kb + 2 * STEP, pA, A);
+        locate(kb + 3 * STEP, pB);
+        consume(kb + STEP, B);
       }
-      // lane holds keys kb + 8*kg + 4*t + r of row j16
-      float bm = -INFINITY;
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = s[t][r] * a.scale;
-          if (edge) {
-            const int key = kb + 8 * kg + 4 * t + r;
-            bool vis = row_ok[rt] && key <= row_pos[rt] && key < ctx;
-            if (a.window > 0) vis = vis && key > row_pos[rt] - a.window;
-            if (!vis) v = -INFINITY;
-          } else if (!row_ok[rt]) {
-            v = -INFINITY;
-          }
-          s[t][r] = v;
-          bm = fmaxf(bm, v);
-        }
-      bm = row_max(bm);
-      const float m_new = fmaxf(m_run[rt], bm);
-      float p[8], corr = 1.f, psum = 0.f;
-      if (m_new == -INFINITY) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) p[e] = 0.f;
-      } else {
-        corr = __expf(m_run[rt] - m_new);  // exp(-inf) = 0 on the first visible block
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            p[4 * t + r] = __expf(s[t][r] - m_new);
-            psum += p[4 * t + r];
-          }
-      }
-      l_run[rt] = l_run[rt] * corr + psum;  // this lane's share of the row's sum
-      m_run[rt] = m_new;
-      typedef __attribute__((ext_vector_type(8))) float f32x8;
-      f32x8 pv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) pv[e] = p[e];
-      const bf16x8 pf = __builtin_convertvector(pv, bf16x8);
-#pragma unroll
-      for (int t = 0; t < DTMAX; ++t)
-        if (t < dt_n) {
-          acc[rt][t] *= corr;
-          acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t], pf, acc[rt][t], 0, 0, 0);
-        }
+    }
+  } else {
+    locate(kb_begin, pA);
+    for (int kb = kb_begin; kb < kb_end; kb += STEP) {
+      fetch(kb, pA, A);
+      locate(kb + STEP, pA);
+      consume(kb, A);
     }
   }
 
-  if (!SPLIT) {
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const float l = row_sum(l_run[rt]);
-      if (!row_ok[rt]) continue;
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      bf16_t* o = out + static_cast<size_t>(q0 + row_tok[rt]) * a.o_stride + row_head[rt] * D + 4 * kg;
-#pragma unroll
-      for (int t = 0; t < DTMAX; ++t)
-        if (t < dt_n) {
-          uint2 pk;
-          pk.x = static_cast<uint32_t>(f32_to_bf16(acc[rt][t][0] * inv)) |
-                 (static_cast<uint32_t>(f32_to_bf16(acc[rt][t][1] * inv)) << 16);
-          pk.y = static_cast<uint32_t>(f32_to_bf16(acc[rt][t][2] * inv)) |
-                 (static_cast<uint32_t>(f32_to_bf16(acc[rt][t][3] * inv)) << 16);
-          *reinterpret_cast<uint2*>(o + t * 16) = pk;
-        }
-    }
-    return;
-  }
-
-  // ---- SPLIT: merge the four waves (RT == 1), then store or hand on the partial result
-  float* red_acc = lds;                                   // [WAVES][dt_n][64][4]
-  float* red_ml = lds + WAVES * dt_n * KVF_WAVE * 4;      // [WAVES][16][2]
+  // ---- merge the four waves, then store or hand on the partial result
+  float* red_acc = lds;                             // [WAVES][DT][64][4]
+  float* red_ml = lds + WAVES * DT * KVF_WAVE * 4;  // [WAVES][16][2]
   const float l_row = row_sum(l_run[0]);
 #pragma unroll
-  for (int t = 0; t < DTMAX; ++t)
-    if (t < dt_n)
-      *reinterpret_cast<f32x4*>(red_acc + ((wave * dt_n + t) * KVF_WAVE + lane) * 4) = acc[0][t];
+  for (int t = 0; t < DT; ++t)
+    *reinterpret_cast<f32x4*>(red_acc + ((wave * DT + t) * KVF_WAVE + lane) * 4) = acc[0][t];
   if (kg == 0) {
-    red_ml[(wave * 16 + j16) * 2] = m_run[0];
+    red_ml[(wave * 16 + j16) * 2] = m_ref[0];
     red_ml[(wave * 16 + j16) * 2 + 1] = l_row;
   }
   __syncthreads();
@@ -285,35 +551,33 @@ __global__ __launch_bounds__(256) void attn_mfma_kernel(
 #pragma unroll
   for (int w = 0; w < WAVES; ++w) {
     const float mw = red_ml[(w * 16 + j16) * 2];
-    cw[w] = mw == -INFINITY ? 0.f : __expf(mw - mm);
+    cw[w] = mw == -INFINITY ? 0.f : exp2f(mw - mm);
     ll += red_ml[(w * 16 + j16) * 2 + 1] * cw[w];
   }
-  if (!row_ok[0]) return;
-  const int head = row_head[0];
-  const size_t slot = (static_cast<size_t>(item_index) * a.H + head) * a.splits + blockIdx.z;
+  if (!rows.ok[0]) return;
+  const int head = rows.head[0];
+  const size_t slot = (static_cast<size_t>(blockIdx.x) * a.H + head) * a.splits + blockIdx.z;
   if (a.splits > 1 && wave == 0 && kg == 0) {
-    part_ml[slot * 2] = mm;
+    part_ml[slot * 2] = mm;  // in log2 units
     part_ml[slot * 2 + 1] = ll;
   }
   const float inv = ll > 0.f ? 1.f / ll : 0.f;
-  for (int t = wave; t < dt_n; t += WAVES) {  // wave w finishes element tiles w, w + 4, ...
+  for (int t = wave; t < DT; t += WAVES) {  // wave w finishes element tiles w, w + 4, ...
     f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < WAVES; ++w)
-      o += *reinterpret_cast<const f32x4*>(red_acc + ((w * dt_n + t) * KVF_WAVE + lane) * 4) * cw[w];
+      o += *reinterpret_cast<const f32x4*>(red_acc + ((w * DT + t) * KVF_WAVE + lane) * 4) * cw[w];
     const int e0 = t * 16 + 4 * kg;
-    if (a.splits == 1) {
-      uint2 pk;
-      pk.x = static_cast<uint32_t>(f32_to_bf16(o[0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[1] * inv)) << 16);
-      pk.y = static_cast<uint32_t>(f32_to_bf16(o[2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(o[3] * inv)) << 16);
-      *reinterpret_cast<uint2*>(out + static_cast<size_t>(q0 + row_tok[0]) * a.o_stride + head * D + e0) = pk;
-    } else {
+    if (a.splits == 1)
+      *reinterpret_cast<uint2*>(out + static_cast<size_t>(q0 + rows.tok[0]) * a.o_stride + head * D + e0) =
+          pack4(o, inv);
+    else
       *reinterpret_cast<f32x4*>(part_acc + slot * D + e0) = o;
-    }
   }
 }
 
-// Merges the splits of every (sequence, head) in split order.  One query token per sequence.
+// Merges the splits of every (sequence, head) in split order.  One query token per sequence;
+// the partial maxima are in log2 units.
 __global__ void attn_split_combine_kernel(const float* __restrict__ part_acc,
                                           const float* __restrict__ part_ml,
                                           const int* __restrict__ seq_ids,
@@ -330,7 +594,7 @@ __global__ void attn_split_combine_kernel(const float* __restrict__ part_acc,
     float ll = 0.f, v = 0.f;
     for (int s = 0; s < splits; ++s) {
       const float ms = part_ml[(slot0 + s) * 2];
-      const float c = ms == -INFINITY ? 0.f : __expf(ms - mm);
+      const float c = ms == -INFINITY ? 0.f : exp2f(ms - mm);
       ll += part_ml[(slot0 + s) * 2 + 1] * c;
       v += part_acc[(slot0 + s) * D + e] * c;
     }
@@ -338,13 +602,52 @@ __global__ void attn_split_combine_kernel(const float* __restrict__ part_acc,
   }
 }
 
-bool args_ok(int H, int KV, int d, int bs) {
-  return d > 0 && d % 16 == 0 && d <= 256 && KV > 0 && H % KV == 0 && bs > 0 && bs % 8 == 0;
+// Also what the 32-bit arithmetic in the kernels needs: positions * page size and the number of
+// 16-byte fragments of a page tensor below 2^32.
+bool args_ok(int H, int KV, int d, int bs, int nb, int table_stride, float scale) {
+  if (!(d > 0 && d % 16 == 0 && d <= 256 && KV > 0 && H % KV == 0 && bs > 0 && bs % 8 == 0)) return false;
+  if (nb < 1 || table_stride < 1 || !(scale > 0.f)) return false;
+  const unsigned long long limit = 1ull << 32;
+  return static_cast<unsigned long long>(table_stride) * bs * bs < limit &&
+         static_cast<unsigned long long>(nb) * KV * bs * d / 8 < limit;
 }
+unsigned magic_of(int bs) { return static_cast<unsigned>((1ull << 32) / bs) + 1u; }
+
+// Row tiles per wave and LDS sharing by head size: what fits the registers and 64 KB of LDS.
+constexpr int runs_rt(int dt) { return dt <= 8 ? 2 : 1; }
+constexpr bool runs_share(int dt) { return dt <= 12; }
+
+template <int DT>
+void launch_runs(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
+                 const int* block_table, const int* work, const int* cu_q, const int* ctx_lens, void* out,
+                 const MArgs& a) {
+  constexpr int RT = runs_rt(DT);
+  constexpr bool SHARE = runs_share(DT);
+  constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
+  const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
+  hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE>), grid, dim3(256), lds, s,
+                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                     static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                     static_cast<bf16_t*>(out), a);
+}
+
+template <int DT>
+void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
+                  const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
+                  void* out, float* part_acc, float* part_ml, const MArgs& a) {
+  const size_t lds = (static_cast<size_t>(WAVES) * DT * KVF_WAVE * 4 + WAVES * 16 * 2) * sizeof(float);
+  hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8)>), grid, dim3(256), lds, s,
+                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                     static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                     static_cast<bf16_t*>(out), part_acc, part_ml, a);
+}
+
+#define KVF_EACH_DT(X) \
+  X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 }  // namespace
 
 // Rows of a query run one workgroup takes: 4 waves x RT tiles x 16 rows.
-KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d) { return d <= 128 ? 128 : 64; }
+KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d) { return WAVES * runs_rt(d / 16) * 16; }
 
 // Query runs: `work` holds num_work pairs (sequence, item) where item i covers rows
 // [i * rows_per_item, (i + 1) * rows_per_item) of the sequence's qlen * H/KV rows per kv head.
@@ -354,19 +657,16 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
                                      int window, int n_seqs, float scale, hipStream_t s) {
   if (num_work <= 0) return 0;
-  if (!args_ok(H, KV, d, bs) || q_stride % 8 != 0 || o_stride % 4 != 0)
+  if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale, magic_of(bs)};
   const dim3 grid(num_work, KV);
-#define GO(DTMAX, RT)                                                                              \
-  hipLaunchKernelGGL((attn_mfma_kernel<DTMAX, RT, false>), grid, dim3(256), 0, s,                  \
-                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),           \
-                     static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,      \
-                     static_cast<bf16_t*>(out), nullptr, nullptr, a)
-  if (d <= 64) GO(4, 2);
-  else if (d <= 128) GO(8, 2);
-  else GO(16, 1);
+  switch (d / 16) {
+#define GO(DT) \
+  case DT: launch_runs<DT>(grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a); break;
+    KVF_EACH_DT(GO)
 #undef GO
+  }
   return kvf_last_error();
 }
 
@@ -380,22 +680,21 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int table_stride, int q_stride, int o_stride, int window,
                                     int n_seqs, int splits, float scale, hipStream_t s) {
   if (num_seqs <= 0) return 0;
-  if (!args_ok(H, KV, d, bs) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
+  if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale};
-  const int G = H / KV, chunks = (G + 15) / 16, dt = d / 16;
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs)};
+  const int G = H / KV, chunks = (G + 15) / 16;
   const dim3 grid(num_seqs, KV * chunks, splits);
-  const size_t lds = (static_cast<size_t>(WAVES) * dt * KVF_WAVE * 4 + WAVES * 16 * 2) * sizeof(float);
-#define GO(DTMAX)                                                                                  \
-  hipLaunchKernelGGL((attn_mfma_kernel<DTMAX, 1, true>), grid, dim3(256), lds, s,                  \
-                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),           \
-                     static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,   \
-                     static_cast<bf16_t*>(out), part_acc, part_ml, a)
-  if (d <= 64) GO(4);
-  else if (d <= 128) GO(8);
-  else GO(16);
+  switch (d / 16) {
+#define GO(DT)                                                                                      \
+  case DT:                                                                                          \
+    launch_split<DT>(grid, s, q, k_pages, vt_pages, block_table, seq_ids, cu_q, ctx_lens, out, part_acc, \
+                     part_ml, a);                                                                   \
+    break;
+    KVF_EACH_DT(GO)
 #undef GO
+  }
   int err = kvf_last_error();
   if (err || splits == 1) return err;
   hipLaunchKernelGGL(attn_split_combine_kernel, dim3(num_seqs, H), dim3(64), 0, s, part_acc,
