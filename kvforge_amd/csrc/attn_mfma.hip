@@ -576,29 +576,35 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_ke
   }
 }
 
-// Merges the splits of every (sequence, head) in split order.  One query token per sequence;
-// the partial maxima are in log2 units.
-__global__ void attn_split_combine_kernel(const float* __restrict__ part_acc,
-                                          const float* __restrict__ part_ml,
-                                          const int* __restrict__ seq_ids,
-                                          const int* __restrict__ cu_q, bf16_t* __restrict__ out,
-                                          int H, int D, int splits, int o_stride, int n_seqs) {
+// Merges the splits of every (sequence, head) in split order.  One query token per sequence, one
+// wave per (sequence, head), at most 64 splits; the partial maxima are in log2 units.  Lane s
+// weighs split s; the loads of the partial accumulators do not depend on one another.
+__global__ __launch_bounds__(64) void attn_split_combine_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    const int* __restrict__ seq_ids, const int* __restrict__ cu_q, bf16_t* __restrict__ out, int H, int D,
+    int splits, int o_stride, int n_seqs) {
   const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
   if (seq < 0 || seq >= n_seqs) return;
-  const int head = blockIdx.y;
+  const int head = blockIdx.y, lane = threadIdx.x;
   const size_t slot0 = (static_cast<size_t>(blockIdx.x) * H + head) * splits;
-  float mm = -INFINITY;
-  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, part_ml[(slot0 + s) * 2]);
+  float m = -INFINITY, l = 0.f;
+  if (lane < splits) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (slot0 + lane) * 2);
+    m = ml.x;
+    l = ml.y;
+  }
   const int tok = cu_q[seq];
-  for (int e = threadIdx.x; e < D; e += blockDim.x) {
-    float ll = 0.f, v = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = part_ml[(slot0 + s) * 2];
-      const float c = ms == -INFINITY ? 0.f : exp2f(ms - mm);
-      ll += part_ml[(slot0 + s) * 2 + 1] * c;
-      v += part_acc[(slot0 + s) * D + e] * c;
-    }
-    out[static_cast<size_t>(tok) * o_stride + head * D + e].bits = f32_to_bf16(ll > 0.f ? v / ll : 0.f);
+  const float mm = wave_max(m);
+  const float c = m == -INFINITY ? 0.f : exp2f(m - mm);
+  const float ll = wave_sum(l * c);
+  const float inv = ll > 0.f ? 1.f / ll : 0.f;
+  for (int e = lane; e < D; e += KVF_WAVE) {
+    float v = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s)
+      v += part_acc[(slot0 + s) * D + e] *
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, c), s));
+    out[static_cast<size_t>(tok) * o_stride + head * D + e].bits = f32_to_bf16(v * inv);
   }
 }
 
@@ -681,7 +687,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int n_seqs, int splits, float scale, hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
-      (splits > 1 && (!part_acc || !part_ml)))
+      splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs)};
   const int G = H / KV, chunks = (G + 15) / 16;

@@ -17,7 +17,8 @@ import numpy as np
 import torch
 
 ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup handles
-DECODE_KEYS_PER_SPLIT = 128
+DECODE_KEYS_PER_SPLIT = 512
+COMPUTE_UNITS = 256
 
 
 @dataclass
@@ -184,12 +185,12 @@ class Step:
         G = H // KV
         chunks = -(-G // 16)
         ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
-        # Few sequences: cut the key range so that a couple of hundred workgroups pull on the
-        # cache, each with at least DECODE_KEYS_PER_SPLIT keys.  Many sequences fill the chip by
-        # themselves; their key range is cut only when it is long.
+        # Few sequences: cut the key range so that about one workgroup per compute unit pulls on
+        # the cache, each cut with at least DECODE_KEYS_PER_SPLIT keys (four key blocks for each
+        # of a workgroup's waves); below that the merge of the cuts costs more than they save.
+        # Many sequences fill the chip by themselves.
         wgs = max(1, self.n_decode * KV * chunks)
-        splits = max(-(-256 // wgs), -(-ctx // 1024))
-        splits = max(1, min(splits, -(-ctx // DECODE_KEYS_PER_SPLIT), 64))
+        splits = max(1, min(COMPUTE_UNITS // wgs, ctx // DECODE_KEYS_PER_SPLIT, 64))
         if splits == 1:
             return 1, None
         acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)

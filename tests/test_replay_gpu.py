@@ -78,9 +78,28 @@ def test_replay_first_tokens_and_one_token_requests(tmp_path):
         ru.compare(folder, tb, out, prompts, *TOL[dtype])
 
 
+def test_replay_decoding_with_split_key_range(tmp_path):
+    """One request decoded past 1,200 tokens: few sequences over a long context make the decode
+    kernel cut the key range into several runs that are merged afterwards."""
+    cfg = dict(ru.TINY_C, max_position_embeddings=2048)
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, cfg, seed=5)
+    ru.sharpen(folder, 6.0)
+    prompts = ru.random_prompts(200, [1240], 11)
+    tb = ru.TraceBuilder()
+    tb.step([("p0", prompts["p0"][:700], [699])])
+    tb.step([("p0", prompts["p0"][700:1200], [499])])
+    for i in range(40):
+        tb.step([("p0", [prompts["p0"][1200 + i]], [0])], end=["p0"] if i == 39 else [])
+    for dtype in ("float32", "bfloat16"):
+        out = str(tmp_path / dtype)
+        ru.run_trace(folder, dtype, tb, out)
+        ru.compare(folder, tb, out, prompts, *TOL[dtype])
+
+
 def test_replay_long_decoding(tmp_path):
-    """Two requests decoded token by token for 300 steps past a short prompt, across many pages
-    and several splits of the decode kernel's key range."""
+    """Two requests decoded token by token for 300 steps past a short prompt, across many
+    pages."""
     folder = str(tmp_path / "model")
     kvforge_amd.write_random_model(folder, ru.TINY_C, seed=3)
     ru.sharpen(folder, 6.0)
