@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512]
-                    [--dtype bfloat16] [--layers L] [--no-points]
+                    [--dtype bfloat16] [--layers L] [--no-points] [--phase all|decode|prefill]
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -117,6 +117,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
+                    help="for profiles: only the decode steps at --batch, or only the prefill")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -136,18 +138,27 @@ def main() -> int:
     with tempfile.TemporaryDirectory(prefix="kvforge_bench_") as folder:
         kvforge_amd.write_random_model(folder, cfg, seed=0)
         results = {}
-        batches = [args.batch] + ([] if args.no_points else [b for b in (1, 64) if b != args.batch])
+        points = args.phase == "all" and not args.no_points
+        batches = [args.batch] + ([b for b in (1, 64) if b != args.batch] if points else [])
+        prefill_s = None
         for b in batches:
             need = b * (args.prompt_len + args.steps + args.warmup + 16)
             engine = build_engine(folder, args.dtype, max(b, 1), max(need, PREFILL_TOKENS + 64),
                                   use_graphs=not args.no_graphs)
-            results[b] = decode_run(engine, vocab, b, args.prompt_len, args.steps, args.warmup)
+            if args.phase != "prefill":
+                results[b] = decode_run(engine, vocab, b, args.prompt_len, args.steps, args.warmup)
             if b == args.batch:
-                prefill_s = prefill_run(engine, vocab, PREFILL_TOKENS)
+                if args.phase != "decode":
+                    prefill_s = prefill_run(engine, vocab, PREFILL_TOKENS)
                 weight_bytes = engine.model.weight_bytes
             del engine
             torch.cuda.empty_cache()
 
+    if args.phase != "all":  # a partial run for a profile: say what was timed and stop
+        part = ({"prefill_ms": round(prefill_s * 1e3, 3)} if args.phase == "prefill" else
+                {"ms_per_step": round(results[args.batch]["ms_per_step"], 4)})
+        print(json.dumps({"phase": args.phase, "batch": args.batch, "dtype": args.dtype, **part}))
+        return 0
     main_run = results[args.batch]
     step_s = main_run["seconds"] / args.steps
     kv_bytes = args.batch * main_run["mean_ctx"] * nums["kv_values_per_token"] * elem
