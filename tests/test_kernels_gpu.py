@@ -261,7 +261,7 @@ class Paged:
     """Scatters contiguous per-sequence K/V into shuffled pages: K ``[nb, KV, bs, d]``, V
     transposed ``[nb, KV, d, bs]``."""
 
-    def __init__(self, seq_lens, KV, d, bs, dtype, seed=0, spare=7):
+    def __init__(self, seq_lens, KV, d, bs, dtype, seed=0, spare=7, shape_keys=None):
         rng = random.Random(seed)
         g = torch.Generator().manual_seed(seed)
         need = sum(-(-n // bs) for n in seq_lens)
@@ -274,7 +274,10 @@ class Paged:
         self.table = torch.full((len(seq_lens), width), -1, dtype=torch.int32)
         self.keys, self.values = [], []
         for s, n in enumerate(seq_lens):
-            kk = torch.randn(n, KV, d, generator=g).to(dtype)
+            kk = torch.randn(n, KV, d, generator=g)
+            if shape_keys is not None:
+                kk = shape_keys(kk)
+            kk = kk.to(dtype)
             vv = torch.randn(n, KV, d, generator=g).to(dtype)
             for b in range(-(-n // bs)):
                 page = ids.pop()
@@ -371,6 +374,43 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     got = out2.float().cpu()
     torch.testing.assert_close(got[[4, 1]], want[[4, 1]], **tol(dtype))
     assert (got[[0, 2, 3, 5]] == 5.0).all()
+
+
+@pytest.mark.parametrize("slope", [0.12, 0.3, -0.2])
+def test_attn_scores_that_keep_rising_or_falling(slope):
+    """Scores that grow (or shrink) steadily with the key's position, by less and by more per key
+    block than the headroom within which the matrix-core kernel leaves its softmax reference
+    alone: a reference raised too late, too early or without rescaling the sums shows here."""
+    H, KV, d, bs, n = 8, 2, 64, 16, 600
+    b16 = torch.bfloat16
+    u = torch.zeros(d)
+    u[3] = 1.0
+
+    def ramp(kk):  # key j gets j * slope * sqrt(d) along u: its score with q = u grows by slope
+        return 0.3 * kk + (torch.arange(kk.shape[0]).float() * slope * math.sqrt(d))[:, None, None] * u
+
+    paged = Paged([n], KV, d, bs, b16, seed=5, shape_keys=ramp)
+    g = torch.Generator().manual_seed(9)
+    q = (0.2 * torch.randn(n, H, d, generator=g) + u).to(b16)
+    scale = 1 / math.sqrt(d)
+    want = plain.causal_attention(q.float(), paged.keys[0].float(), paged.values[0].float(), scale, 0)
+    want = want.reshape(n, H * d)
+    cu = torch.tensor([0, n], dtype=torch.int32)
+    ctx = torch.tensor([n], dtype=torch.int32)
+    out = torch.zeros(n, H * d, dtype=b16, device=DEV)
+    ops().attn_prefill(q.reshape(n, H * d).to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                       cu.to(DEV), ctx.to(DEV), prefill_work([n], H // KV, b16, d, bs).to(DEV), out,
+                       H, KV, d, scale, 0)
+    torch.testing.assert_close(out.float().cpu(), want, atol=2e-2, rtol=2e-2)
+    # the last token alone, through the decode kernel, whole and in cuts
+    cu1 = torch.tensor([0, 1], dtype=torch.int32)
+    for splits in (1, 3):
+        ws = (torch.empty(H * splits * d, device=DEV), torch.empty(H * splits * 2, device=DEV))
+        one = torch.zeros(1, H * d, dtype=b16, device=DEV)
+        ops().attn_decode(q[n - 1:].reshape(1, H * d).to(DEV), paged.k.to(DEV), paged.v.to(DEV),
+                          paged.table.to(DEV), None, 1, cu1.to(DEV), ctx.to(DEV), one, H, KV, d, scale,
+                          0, splits, ws)
+        torch.testing.assert_close(one.float().cpu(), want[n - 1:], atol=2e-2, rtol=2e-2)
 
 
 def test_attn_far_key_stands_out():
