@@ -62,18 +62,95 @@ __device__ __forceinline__ bf16x8 load_frag_f32(const float* p, bool ok, float& 
   return __builtin_convertvector(x, bf16x8);
 }
 
+// What an epilogue reads besides the accumulators.  With one row tile the lanes of wave 0 finish
+// the workgroup's tile and know their row and columns from the start, so they ask for these
+// operands before the walk over K and find them in registers afterwards, instead of paying
+// their latencies (up to three dependent loads for the cache write) at the end.
+struct EpiOperands {
+  f32x4 c;            // EPI 2: the four values the product is added to
+  int pos, page;      // EPI 4: the token's position; the page its key and value go to (or -1)
+  float cs[2], sn[2]; // EPI 4: rotation of the lane's two pairs
+  bool have;
+};
+
+// 16-byte accesses to C are possible where rows and base are aligned and all four columns exist
+__device__ __forceinline__ bool vec4_ok(const void* Cv, int ldc, int n, int N, int elem) {
+  return n + 3 < N && (ldc * elem) % 16 == 0 && n % 4 == 0 &&
+         reinterpret_cast<uintptr_t>(Cv) % 16 == 0;
+}
+
+// First stage: loads that need only (m, n).
+template <int EPI>
+__device__ __forceinline__ void epi_prefetch_a(EpiOperands& op, int m, int n, int N, int ldc, const void* Cv,
+                                               const RopeEpi& rp) {
+  op.have = true;
+  if (EPI == 2) {
+    const float* c = static_cast<const float*>(Cv) + static_cast<size_t>(m) * ldc + n;
+    if (vec4_ok(Cv, ldc, n, N, 4)) {
+      op.c = *reinterpret_cast<const f32x4*>(c);
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) op.c[r] = n + r < N ? c[r] : 0.f;
+    }
+  }
+  if (EPI == 4) {
+    op.pos = rp.positions[m];
+    op.page = rp.write_kv ? rp.seq_of_token[m] : -1;  // the sequence for now
+  }
+}
+// Second stage: loads that need what the first brought (position -> angles, sequence -> page).
+template <int EPI>
+__device__ __forceinline__ void epi_prefetch_b(EpiOperands& op, int n, const RopeEpi& rp) {
+  if (EPI != 4) return;
+  const int head = n / rp.d, e = n - head * rp.d;
+  const int p = op.pos;
+  const bool pos_ok = p >= 0 && p < rp.table_len;
+#pragma unroll
+  for (int pr = 0; pr < 2; ++pr) {
+    const int j = (e + 2 * pr) / 2;
+    const bool rotate = head < rp.H + rp.KV && pos_ok && 2 * j + 1 < rp.rot;
+    op.cs[pr] = rotate ? rp.cos_t[static_cast<size_t>(p) * (rp.rot / 2) + j] : 1.f;
+    op.sn[pr] = rotate ? rp.sin_t[static_cast<size_t>(p) * (rp.rot / 2) + j] : 0.f;
+  }
+  const int seq = op.page;
+  int page = -1;
+  if (head >= rp.H && rp.write_kv && pos_ok) {
+    const int blk = p / rp.block_size;
+    if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
+      page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
+  }
+  op.page = page;
+}
+
 // One lane's four neighbouring columns n..n+3 of row m, after the waves' partial sums are added.
 template <int EPI>
 __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, int ldc, void* Cv,
-                                           const RopeEpi& rp) {
+                                           const RopeEpi& rp, EpiOperands& op) {
+  if (EPI == 2 || EPI == 4) {
+    if (!op.have) {
+      epi_prefetch_a<EPI>(op, m, n, N, ldc, Cv, rp);
+      epi_prefetch_b<EPI>(op, n, rp);
+    }
+  }
   if (EPI <= 2) {
+    const size_t idx = static_cast<size_t>(m) * ldc + n;
+    if (EPI == 0 && vec4_ok(Cv, ldc, n, N, 4)) {
+      *reinterpret_cast<f32x4*>(static_cast<float*>(Cv) + idx) = s;
+    } else if (EPI == 2 && vec4_ok(Cv, ldc, n, N, 4)) {
+      *reinterpret_cast<f32x4*>(static_cast<float*>(Cv) + idx) = op.c + s;
+    } else if (EPI == 1 && vec4_ok(Cv, ldc, n, N, 2)) {
+      uint2 packed;
+      packed.x = static_cast<uint32_t>(f32_to_bf16(s[0])) | (static_cast<uint32_t>(f32_to_bf16(s[1])) << 16);
+      packed.y = static_cast<uint32_t>(f32_to_bf16(s[2])) | (static_cast<uint32_t>(f32_to_bf16(s[3])) << 16);
+      *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + idx) = packed;
+    } else {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      if (n + r >= N) break;
-      const size_t idx = static_cast<size_t>(m) * ldc + n + r;
-      if (EPI == 0) static_cast<float*>(Cv)[idx] = s[r];
-      if (EPI == 1) static_cast<bf16_t*>(Cv)[idx].bits = f32_to_bf16(s[r]);
-      if (EPI == 2) static_cast<float*>(Cv)[idx] += s[r];
+      for (int r = 0; r < 4; ++r) {
+        if (n + r >= N) break;
+        if (EPI == 0) static_cast<float*>(Cv)[idx + r] = s[r];
+        if (EPI == 1) static_cast<bf16_t*>(Cv)[idx + r].bits = f32_to_bf16(s[r]);
+        if (EPI == 2) static_cast<float*>(Cv)[idx + r] = op.c[r] + s[r];
+      }
     }
   } else if (EPI == 3) {
     // N is even and n a multiple of 4: two (gate, up) pairs
@@ -81,50 +158,36 @@ __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, 
     o[0].bits = f32_to_bf16(s[0] / (1.f + __expf(-s[0])) * s[1]);
     if (n + 2 < N) o[1].bits = f32_to_bf16(s[2] / (1.f + __expf(-s[2])) * s[3]);
   } else {
-    // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head
+    // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head; pairs
+    // that are not rotated (v heads, elements past the rotary width, positions off the table)
+    // carry the identity
     const int head = n / rp.d, e = n - head * rp.d;
-    const int p = rp.positions[m];
-    const bool pos_ok = p >= 0 && p < rp.table_len;
-    float o[4] = {s[0], s[1], s[2], s[3]};
-    if (head < rp.H + rp.KV && pos_ok) {
+    float o[4];
 #pragma unroll
-      for (int pr = 0; pr < 2; ++pr) {
-        const int j = (e + 2 * pr) / 2;
-        if (2 * j + 1 < rp.rot) {
-          const float c = rp.cos_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
-          const float sn = rp.sin_t[static_cast<size_t>(p) * (rp.rot / 2) + j];
-          const float x1 = s[2 * pr], x2 = s[2 * pr + 1];
-          o[2 * pr] = x1 * c - x2 * sn;
-          o[2 * pr + 1] = x2 * c + x1 * sn;
-        }
-      }
+    for (int pr = 0; pr < 2; ++pr) {
+      const float x1 = s[2 * pr], x2 = s[2 * pr + 1];
+      o[2 * pr] = x1 * op.cs[pr] - x2 * op.sn[pr];
+      o[2 * pr + 1] = x2 * op.cs[pr] + x1 * op.sn[pr];
     }
     uint2 packed;
     packed.x = static_cast<uint32_t>(f32_to_bf16(o[0])) | (static_cast<uint32_t>(f32_to_bf16(o[1])) << 16);
     packed.y = static_cast<uint32_t>(f32_to_bf16(o[2])) | (static_cast<uint32_t>(f32_to_bf16(o[3])) << 16);
     if (head < rp.H) {
       *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n) = packed;
-    } else if (rp.write_kv && pos_ok) {
-      const int seq = rp.seq_of_token[m];
-      const int blk = p / rp.block_size;
-      int page = -1;
-      if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
-        page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
-      if (page >= 0 && page < rp.num_blocks) {
-        const int off = p - blk * rp.block_size;
-        if (head < rp.H + rp.KV) {
-          const int kvh = head - rp.H;
-          *reinterpret_cast<uint2*>(
-              rp.k_pages + ((static_cast<size_t>(page) * rp.KV + kvh) * rp.block_size + off) * rp.d +
-              e) = packed;
-        } else {
-          // V pages are [num_blocks, KV, d, block_size]: one element per key row
-          const int kvh = head - rp.H - rp.KV;
-          bf16_t* dst = rp.v_pages +
-                        ((static_cast<size_t>(page) * rp.KV + kvh) * rp.d + e) * rp.block_size + off;
+    } else if (op.page >= 0 && op.page < rp.num_blocks) {
+      const int off = op.pos % rp.block_size;
+      if (head < rp.H + rp.KV) {
+        const int kvh = head - rp.H;
+        *reinterpret_cast<uint2*>(
+            rp.k_pages + ((static_cast<size_t>(op.page) * rp.KV + kvh) * rp.block_size + off) * rp.d + e) =
+            packed;
+      } else {
+        // V pages are [num_blocks, KV, d, block_size]: one element per key row
+        const int kvh = head - rp.H - rp.KV;
+        bf16_t* dst =
+            rp.v_pages + ((static_cast<size_t>(op.page) * rp.KV + kvh) * rp.d + e) * rp.block_size + off;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) dst[static_cast<size_t>(r) * rp.block_size].bits = f32_to_bf16(o[r]);
-        }
+        for (int r = 0; r < 4; ++r) dst[static_cast<size_t>(r) * rp.block_size].bits = f32_to_bf16(o[r]);
       }
     }
   }
@@ -177,9 +240,24 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
     for (int j = 0; j < NT; ++j) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  // With one row tile, lane l of wave 0 will finish C[m_base + l%16][n0 + j*RW + 4*(l/16) ..+3]:
+  // it asks for what its epilogue reads now, and for what depends on that after its first pass.
+  constexpr bool PRE = MT == 1 && (EPI == 2 || EPI == 4);
+  EpiOperands pre[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) pre[j].have = false;
+  const int pre_m = m_base + r16, pre_n = n0 + 4 * kg;
+  const bool pre_mine = PRE && wave == 0 && pre_m < M && 4 * kg < RW;
+  if (pre_mine) {
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      if (pre_n + j * RW < N) epi_prefetch_a<EPI>(pre[j], pre_m, pre_n + j * RW, N, ldc, Cv, rp);
+  }
+
   const int ksteps = (K + 31) / 32;
-  int ks = wave;
   constexpr int U = depth(MT, NT, AT);
+  int ks = wave;
+  bool first = true;
   for (; ks + (U - 1) * nw < ksteps; ks += U * nw) {
     bf16x8 wf[U][NT], af[U][MT];
 #pragma unroll
@@ -199,6 +277,19 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 #pragma unroll
         for (int t = 0; t < MT; ++t)
           acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][j], af[u][t], acc[j][t], 0, 0, 0);
+    if (PRE && first) {  // the first stage has arrived with this pass's loads
+      first = false;
+      if (pre_mine) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          if (pre[j].have) epi_prefetch_b<EPI>(pre[j], pre_n + j * RW, rp);
+      }
+    }
+  }
+  if (PRE && first && pre_mine) {  // K too short for a full pass
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      if (pre[j].have) epi_prefetch_b<EPI>(pre[j], pre_n + j * RW, rp);
   }
   for (; ks < ksteps; ks += nw) {
     const int k = ks * 32;
@@ -246,7 +337,9 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
         for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
         s *= rsqrtf(tot / static_cast<float>(K) + eps);
       }
-      store_tile<EPI>(s, m, n, N, ldc, Cv, rp);
+      EpiOperands fresh;
+      fresh.have = false;
+      store_tile<EPI>(s, m, n, N, ldc, Cv, rp, PRE ? pre[j] : fresh);
     }
   }
 }
@@ -254,12 +347,11 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 int g_waves_override = 0;
 int g_rows_override = 0;
 
-// Waves per workgroup, as measured on the shapes of a 1B-parameter decoder: eight when the grid
-// is small (fewer leave loads unhidden, sixteen crowd the CU), four when a thousand or more
-// workgroups already fill every CU several times; at least one k-step per wave.
-int pick_waves(int groups, int K) {
+// Waves per workgroup, as measured on the shapes of a 1B-parameter decoder: eight (fewer leave
+// loads unhidden, sixteen crowd the CU); at least one k-step per wave.
+int pick_waves(int K) {
   const int ksteps = (K + 31) / 32;
-  int nw = g_waves_override > 0 ? g_waves_override : (groups >= 1024 ? 4 : 8);
+  int nw = g_waves_override > 0 ? g_waves_override : 8;
   if (nw > 16) nw = 16;
   if (nw > ksteps) nw = ksteps;
   if (nw < 1) nw = 1;
@@ -270,7 +362,7 @@ template <int MT, int NT, int AT, int EPI, int RW = 16>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
                int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
   const int groups = (N + RW * NT - 1) / (RW * NT);
-  int nw = pick_waves(groups, K);
+  int nw = pick_waves(K);
   if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
   const dim3 grid(groups), block(nw * KVF_WAVE);
   const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
@@ -292,9 +384,13 @@ int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int 
       return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
   }
   if (MT == 1) {
-    const int rw = g_rows_override > 0 ? g_rows_override : 16;  // fewer rows measured no gain
+    // Every workgroup reads all of A, so with several rows of A and many rows of W a workgroup
+    // takes 32 rows of W and halves that traffic; fewer than 16 rows measured no gain anywhere.
+    const int rw = g_rows_override > 0 ? g_rows_override : (M - m_base > 4 && tiles >= 512 ? 32 : 16);
     if (rw == 4) return launch_one<1, 1, AT, EPI, 4>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
     if (rw == 8) return launch_one<1, 1, AT, EPI, 8>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
   }
   return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
 }
