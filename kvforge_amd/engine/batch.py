@@ -18,6 +18,7 @@ import torch
 
 ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup handles
 DECODE_KEYS_PER_SPLIT = 512
+MAX_DECODE_SPLITS = 64  # what the merge kernel takes (one lane per cut)
 COMPUTE_UNITS = 256
 
 
@@ -190,7 +191,7 @@ class Step:
         # of a workgroup's waves); below that the merge of the cuts costs more than they save.
         # Many sequences fill the chip by themselves.
         wgs = max(1, self.n_decode * KV * chunks)
-        splits = max(1, min(COMPUTE_UNITS // wgs, ctx // DECODE_KEYS_PER_SPLIT, 64))
+        splits = max(1, min(COMPUTE_UNITS // wgs, ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS))
         if splits == 1:
             return 1, None
         acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)

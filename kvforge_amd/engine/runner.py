@@ -16,7 +16,8 @@ import torch
 
 from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
-from kvforge_amd.engine.batch import MetaBuffers, Step, StepEntry, Workspace, fill_step
+from kvforge_amd.engine.batch import (DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS, MetaBuffers, Step, StepEntry,
+                                      Workspace, fill_step)
 from kvforge_amd.kernels import ops
 from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
@@ -119,10 +120,11 @@ class ModelRunner:
             bucket *= 2
         bucket = min(bucket, self.meta.max_seqs)
         step, _ = self.build_step(entries, pad_to=bucket)
-        ctx_bucket = 256
-        while ctx_bucket < step.max_decode_ctx:
-            ctx_bucket *= 2
-        step.max_decode_ctx = ctx_bucket
+        # The longest context enters the captured launches only through the number of cuts of
+        # the key range, which grows by one per DECODE_KEYS_PER_SPLIT keys up to a limit: graphs
+        # are kept per such cell, planned for the cell's lower edge.
+        ctx_bucket = min(step.max_decode_ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
+        step.max_decode_ctx = max(ctx_bucket * DECODE_KEYS_PER_SPLIT, 1)
         cap = self.meta.max_seqs
         fh, ih = self._sample_f_np, self._sample_i_np
         ids = [e.request_id for e in entries]
