@@ -35,10 +35,29 @@ KVF_EXPORT int kvf_embed_bf16(const int* ids, const void* t, float* o, int n, in
 // y = x * rsqrt(mean(x^2) + eps) * w, all in fp32, rounded once to T on store.
 // x is the fp32 residual stream; `rows` (may be null) gathers input rows; w is fp32 or T, or
 // null when the weight has been folded into the matrix that consumes y.
+// `delta` (may be null, [x_rows, h] of T) is a sum still owed to the stream: the norm is taken of
+// x + delta, and without `rows` the sum is also written back to x, which saves the pass of an
+// add kernel of its own.
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4(float* p, const float4& v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, const float4& v) {
+  uint2 r;
+  r.x = static_cast<uint32_t>(f32_to_bf16(v.x)) | (static_cast<uint32_t>(f32_to_bf16(v.y)) << 16);
+  r.y = static_cast<uint32_t>(f32_to_bf16(v.z)) | (static_cast<uint32_t>(f32_to_bf16(v.w)) << 16);
+  *reinterpret_cast<uint2*>(p) = r;
+}
+
+constexpr int NORM_KEEP = 4;  // float4s a thread keeps in registers between the two passes
+
 template <typename T, typename W>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
-                               const W* __restrict__ w, float eps, T* __restrict__ out, int h,
-                               int x_rows) {
+__global__ void rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ rows,
+                               const T* __restrict__ delta, const W* __restrict__ w, float eps,
+                               T* __restrict__ out, int h, int x_rows, int aligned) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
   int src = rows ? rows[m] : m;
@@ -47,42 +66,107 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const int* __restric
     for (int i = threadIdx.x; i < h; i += blockDim.x) Elem<T>::store(o + i, 0.f);
     return;
   }
-  const float* xr = x + static_cast<size_t>(src) * h;
+  float* xr = x + static_cast<size_t>(src) * h;
+  const T* dr = delta ? delta + static_cast<size_t>(src) * h : nullptr;
+  const bool write_back = dr && !rows;
   float ss = 0.f;
+  if (aligned && h <= static_cast<int>(blockDim.x) * 4 * NORM_KEEP) {
+    // the row stays in registers: one read of x (and delta), one write of y (and x)
+    float4 v[NORM_KEEP];
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; ++k) {
+      const int i = (k * blockDim.x + threadIdx.x) * 4;
+      v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (i < h) {
+        v[k] = load4(xr + i);
+        if (dr) {
+          const float4 d = load4(dr + i);
+          v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+          if (write_back) store4(xr + i, v[k]);
+        }
+        ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+      }
+    }
+    ss = block_sum(ss, scratch);
+    const float r = rsqrtf(ss / static_cast<float>(h) + eps);
+#pragma unroll
+    for (int k = 0; k < NORM_KEEP; ++k) {
+      const int i = (k * blockDim.x + threadIdx.x) * 4;
+      if (i < h) {
+        float4 y = make_float4(v[k].x * r, v[k].y * r, v[k].z * r, v[k].w * r);
+        if (w) {
+          const float4 g = load4(w + i);
+          y.x *= g.x; y.y *= g.y; y.z *= g.z; y.w *= g.w;
+        }
+        store4(o + i, y);
+      }
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
-    const float v = xr[i];
+    float v = xr[i];
+    if (dr) {
+      v += Elem<T>::load(dr + i);
+      if (write_back) xr[i] = v;
+    }
     ss += v * v;
   }
   ss = block_sum(ss, scratch);
   const float r = rsqrtf(ss / static_cast<float>(h) + eps);
-  if (w) {
-    for (int i = threadIdx.x; i < h; i += blockDim.x)
-      Elem<T>::store(o + i, xr[i] * r * Elem<W>::load(w + i));
-  } else {
-    for (int i = threadIdx.x; i < h; i += blockDim.x) Elem<T>::store(o + i, xr[i] * r);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    float v = xr[i];  // already the sum where it was written back (by this same thread)
+    if (dr && !write_back) v += Elem<T>::load(dr + i);
+    Elem<T>::store(o + i, w ? v * r * Elem<W>::load(w + i) : v * r);
   }
 }
 
 template <typename T>
-static int rmsnorm_launch(const float* x, const int* rows, const void* w, int w_is_f32, float eps,
-                          void* out, int m, int h, int x_rows, hipStream_t s) {
+static int rmsnorm_launch(float* x, const int* rows, const void* delta, const void* w, int w_is_f32,
+                          float eps, void* out, int m, int h, int x_rows, hipStream_t s) {
   if (m <= 0) return 0;
   const int threads = h >= 1024 ? 256 : (h >= 256 ? 128 : 64);
+  auto at = [](const void* p, size_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; };
+  const int aligned = h % 4 == 0 && at(x, 16) && at(out, 4 * sizeof(T)) && at(delta, 4 * sizeof(T)) &&
+                      at(w, w_is_f32 ? 16 : 4 * sizeof(T));
   if (w_is_f32)
     hipLaunchKernelGGL((rmsnorm_kernel<T, float>), dim3(m), dim3(threads), 0, s, x, rows,
-                       static_cast<const float*>(w), eps, static_cast<T*>(out), h, x_rows);
+                       static_cast<const T*>(delta), static_cast<const float*>(w), eps,
+                       static_cast<T*>(out), h, x_rows, aligned);
   else
     hipLaunchKernelGGL((rmsnorm_kernel<T, T>), dim3(m), dim3(threads), 0, s, x, rows,
-                       static_cast<const T*>(w), eps, static_cast<T*>(out), h, x_rows);
+                       static_cast<const T*>(delta), static_cast<const T*>(w), eps,
+                       static_cast<T*>(out), h, x_rows, aligned);
   return kvf_last_error();
 }
-KVF_EXPORT int kvf_rmsnorm_f32(const float* x, const int* rows, const void* w, int wf, float eps,
-                               void* out, int m, int h, int xr, hipStream_t s) {
-  return rmsnorm_launch<float>(x, rows, w, wf, eps, out, m, h, xr, s);
+KVF_EXPORT int kvf_rmsnorm_f32(float* x, const int* rows, const void* delta, const void* w, int wf,
+                               float eps, void* out, int m, int h, int xr, hipStream_t s) {
+  return rmsnorm_launch<float>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
 }
-KVF_EXPORT int kvf_rmsnorm_bf16(const float* x, const int* rows, const void* w, int wf, float eps,
-                                void* out, int m, int h, int xr, hipStream_t s) {
-  return rmsnorm_launch<bf16_t>(x, rows, w, wf, eps, out, m, h, xr, s);
+KVF_EXPORT int kvf_rmsnorm_bf16(float* x, const int* rows, const void* delta, const void* w, int wf,
+                                float eps, void* out, int m, int h, int xr, hipStream_t s) {
+  return rmsnorm_launch<bf16_t>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
+}
+
+// ----------------------------------------------------------------------------- residual sum
+// x[m] += delta[m] in fp32 (x is the residual stream, delta a product in T).
+template <typename T>
+__global__ void add_rows_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t total) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < total) x[i] += Elem<T>::load(delta + i);
+}
+template <typename T>
+static int add_rows_launch(float* x, const void* delta, int m, int h, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * h;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(add_rows_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s,
+                     x, static_cast<const T*>(delta), total);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_add_rows_f32(float* x, const void* d, int m, int h, hipStream_t s) {
+  return add_rows_launch<float>(x, d, m, h, s);
+}
+KVF_EXPORT int kvf_add_rows_bf16(float* x, const void* d, int m, int h, hipStream_t s) {
+  return add_rows_launch<bf16_t>(x, d, m, h, s);
 }
 
 // ----------------------------------------------------------------------------- SwiGLU gate
@@ -101,11 +185,34 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   const float u = Elem<T>::load(paired ? row + 2 * i + 1 : row + inter + i);
   Elem<T>::store(out + idx, g / (1.f + expf(-g)) * u);
 }
+// bf16, paired: a thread takes four neighbouring (gate, up) pairs (16 bytes in, 8 bytes out)
+__global__ void silu_mul_pairs4_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                       size_t quads) {
+  const size_t q = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (q >= quads) return;
+  float v[8];
+  load8(gu + q * 8, v);
+  uint2 packed;
+  uint32_t h[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) h[i] = f32_to_bf16(v[2 * i] / (1.f + __expf(-v[2 * i])) * v[2 * i + 1]);
+  packed.x = h[0] | (h[1] << 16);
+  packed.y = h[2] | (h[3] << 16);
+  *reinterpret_cast<uint2*>(out + q * 4) = packed;
+}
+
 template <typename T>
 static int silu_mul_launch(const void* gu, void* out, int m, int inter, int paired,
                            hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * inter;
   if (total == 0) return 0;
+  if (sizeof(T) == 2 && paired && inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+    const size_t quads = total / 4;
+    hipLaunchKernelGGL(silu_mul_pairs4_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256),
+                       0, s, static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), quads);
+    return kvf_last_error();
+  }
   const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
   hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, s,
                      static_cast<const T*>(gu), static_cast<T*>(out), inter, total, paired);

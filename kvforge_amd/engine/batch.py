@@ -154,6 +154,32 @@ class Step:
         self._work: dict[tuple[int, int], torch.Tensor | None] = {}
         self._identity_rotary = None
         self.device: torch.device | str = "cuda"
+        # A product still owed to the residual stream: (stream, product).  A part that ends in a
+        # library product over many rows leaves it here instead of running an add kernel; the
+        # next norm adds it on its way (``take_owed``), anything else calls ``settle`` first.
+        self.owed: tuple[torch.Tensor, torch.Tensor] | None = None
+
+    def owe(self, residual: torch.Tensor, product: torch.Tensor) -> None:
+        self.settle()
+        self.owed = (residual, product)
+
+    def take_owed(self, residual: torch.Tensor) -> torch.Tensor | None:
+        """The product owed to ``residual``, for a norm kernel that adds it itself."""
+        if self.owed is None:
+            return None
+        if self.owed[0] is not residual:
+            self.settle()
+            return None
+        product = self.owed[1]
+        self.owed = None
+        return product
+
+    def settle(self) -> None:
+        """Add what is owed to the residual stream now."""
+        if self.owed is not None:
+            from kvforge_amd.kernels import ops
+            ops.add_rows(*self.owed)
+            self.owed = None
 
     def prefill_work(self, group_size: int, rows_per_item: int = ROWS_PER_TILE
                      ) -> torch.Tensor | None:

@@ -88,9 +88,11 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
 
 # ------------------------------------------------------------------------------ RMS norm
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch.Tensor,
-            rows: torch.Tensor | None = None) -> None:
-    """``out[m] = x[rows[m] or m] * rsqrt(mean(x^2) + eps) * weight`` with fp32 math
-    (``weight=None``: no weight, for a norm whose weight is folded into the next matrix)."""
+            rows: torch.Tensor | None = None, add: torch.Tensor | None = None) -> None:
+    """``out[m] = y * rsqrt(mean(y^2) + eps) * weight`` with ``y = x[rows[m] or m]`` in fp32
+    (``weight=None``: no weight, for a norm whose weight is folded into the next matrix).
+    ``add`` (``[rows of x, h]``, dtype of ``out``) is a sum still owed to ``x``: the norm is taken
+    of ``x + add``, and without ``rows`` the sum is written back to ``x`` as well."""
     _check(x, "x", F32, (None, None))
     xr, h = x.shape
     m = out.shape[0]
@@ -103,12 +105,24 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch
         _check(rows, "rows", I32, (m,))
     elif m > xr:
         raise KernelError("rmsnorm: more output rows than input rows")
+    if add is not None:
+        _check(add, "add", out.dtype, (xr, h))
     f = _fn("elementwise", f"kvf_rmsnorm_{_suffix(out.dtype)}",
-            [c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p])
+            [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int,
+             c_void_p])
     _ok(f(x.data_ptr(), rows.data_ptr() if rows is not None else None,
+          add.data_ptr() if add is not None else None,
           weight.data_ptr() if weight is not None else None,
           1 if weight is not None and weight.dtype == F32 else 0, float(eps), out.data_ptr(),
           m, h, xr, _stream()), "rmsnorm")
+
+
+def add_rows(x: torch.Tensor, delta: torch.Tensor) -> None:
+    """``x += delta`` for the fp32 residual stream ``x`` and a product ``delta`` of equal shape."""
+    _check(x, "x", F32, (None, None))
+    _check(delta, "delta", None, tuple(x.shape))
+    f = _fn("elementwise", f"kvf_add_rows_{_suffix(delta.dtype)}", [c_void_p, c_void_p, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), delta.data_ptr(), x.shape[0], x.shape[1], _stream()), "add_rows")
 
 
 # ------------------------------------------------------------------------------ SwiGLU gate
@@ -198,6 +212,14 @@ def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False) -> bo
     lda = a.stride(0) if m > 1 else k
     return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and k % 8 == 0 and lda % 8 == 0
             and m <= (FUSED_NORM_MAX_M if rms else SKINNY_MAX_M))
+
+
+def is_library_product(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm(a, w, ...)`` hands the product to the library (bf16, more rows than the
+    weight-streaming kernel takes)."""
+    m, k = a.shape
+    lda = a.stride(0) if m > 1 else k
+    return (a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0 and m > SKINNY_MAX_M)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:

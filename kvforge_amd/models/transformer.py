@@ -107,9 +107,11 @@ class Transformer:
             spec.blocks[call.layer].forward(residual, step, ls)
         r = step.n_logits
         if r == 0:
+            step.owed = None
             return torch.empty((0, cfg.vocab_size), dtype=torch.float32, device=residual.device)
         x = step.ws.buf("final_normed", (r, hidden), step.act_dtype)
-        spec.final_norm.forward(residual, x, step.logits_rows)
+        # only the wanted rows matter now: what is still owed to the stream is added to them alone
+        spec.final_norm.forward(residual, x, step.logits_rows, add=step.take_owed(residual))
         logits = step.ws.buf("logits", (r, cfg.vocab_size), torch.float32)
         spec.head.forward(x, logits)
         return logits

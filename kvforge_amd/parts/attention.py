@@ -13,7 +13,7 @@ import math
 import torch
 
 from kvforge_amd.kernels import ops
-from kvforge_amd.parts.base import CacheSpec, LayerState, Mixer, WeightSpec
+from kvforge_amd.parts.base import CacheSpec, LayerState, Mixer, WeightSpec, add_product
 from kvforge_amd.parts.positions import RotaryPositions
 from kvforge_amd.registry import register_mixer
 
@@ -21,6 +21,8 @@ from kvforge_amd.registry import register_mixer
 @register_mixer("attention")
 class PagedAttention(Mixer):
     """``window``: ``None`` attends to every earlier position, ``w`` to the last ``w``."""
+
+    settles_residual = True  # its norm kernel adds what is owed to the stream
 
     def __init__(self, prefix: str, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary: RotaryPositions | None, scale: float | None = None,
@@ -99,10 +101,13 @@ class PagedAttention(Mixer):
         cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else step.no_rotation()
         rms = self.norm_eps
         if rms is not None and not ops.bf16_kernel_takes(x, self.w_qkv, True):
-            # too many rows for the norm to ride in the projection: a norm kernel of its own
+            # too many rows for the norm to ride in the projection: a norm kernel of its own,
+            # which also adds what the layer before still owes the stream
             normed = ws.buf("normed", (n, self.hidden), act)
-            ops.rmsnorm(x, None, rms, normed)
+            ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
+        else:
+            step.settle()
         if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None) and layer.k_pages.dtype == torch.bfloat16:
             # one kernel: (norm,) projection, rotary, cache write
             qkv = ws.buf("q_rot", (n, H * d), act)
@@ -126,4 +131,4 @@ class PagedAttention(Mixer):
             ops.attn_decode(qkv, layer.k_pages, layer.v_pages, table, step.decode_seq_ids,
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace)
-        ops.gemm(out, self.w_o, residual, accumulate=True)
+        add_product(step, out, self.w_o, residual)

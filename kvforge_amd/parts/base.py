@@ -93,8 +93,11 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
-        """``out[m] = norm(x[rows[m] or m])``; ``x`` is the fp32 residual stream."""
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None,
+                add: torch.Tensor | None = None) -> None:
+        """``out[m] = norm(x[rows[m] or m])``; ``x`` is the fp32 residual stream.  ``add`` is a
+        product still owed to ``x`` (same shape): the norm is taken of ``x + add``, and without
+        ``rows`` the sum is left in ``x``."""
         raise NotImplementedError
 
 
@@ -110,7 +113,13 @@ class Positions(Part):
 
 
 class Mixer(Part):
-    """Mixes information across the tokens of a sequence (attention, recurrences, ...)."""
+    """Mixes information across the tokens of a sequence (attention, recurrences, ...).
+
+    ``settles_residual``: a part that sets this looks after ``step.owed`` itself (it takes the
+    owed product into its norm kernel); every other part is handed a residual stream that is
+    up to date."""
+
+    settles_residual = False
 
     cache_spec: CacheSpec | None = None
     state_spec: StateSpec | None = None
@@ -122,6 +131,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    settles_residual = False
+
     def forward(self, x: torch.Tensor, step: "Step", residual: torch.Tensor) -> None:
         """Add the feed-forward output for ``x [N, hidden]`` into ``residual`` (fp32)."""
         raise NotImplementedError
@@ -156,6 +167,21 @@ class Block(Part):
 
     def num_bytes(self) -> int:
         return sum(p.num_bytes() for p in self.parts())
+
+
+def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor) -> None:
+    """``residual += a @ w.T``, the last product of a mixer or feed-forward.  With few rows (or in
+    fp32) the product kernel adds in its epilogue.  Many bf16 rows go to the library, whose
+    product is left owed to the stream (``step.owe``) so that the next norm adds it on its way
+    instead of an add kernel of its own."""
+    from kvforge_amd.kernels import ops
+
+    if ops.is_library_product(a, w):
+        product = step.ws.buf("owed_product", (a.shape[0], w.shape[0]), a.dtype)
+        ops.gemm(a, w, product)
+        step.owe(residual, product)
+    else:
+        ops.gemm(a, w, residual, accumulate=True)
 
 
 @dataclass(frozen=True)

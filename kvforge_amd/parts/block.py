@@ -26,14 +26,18 @@ class PreNormBlock(Block):
 
     def forward(self, residual, step, layer: LayerState) -> None:
         if self.mixer_takes_residual:
+            if not self.mixer.settles_residual:
+                step.settle()
             self.mixer.forward(residual, step, layer, residual)
         else:
             x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
-            self.mixer_norm.forward(residual, x)
+            self.mixer_norm.forward(residual, x, add=step.take_owed(residual))
             self.mixer.forward(x, step, layer, residual)
         if self.ffn_takes_residual:
+            if not self.ffn.settles_residual:
+                step.settle()
             self.ffn.forward(residual, step, residual)
         else:
             x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
-            self.ffn_norm.forward(residual, x)
+            self.ffn_norm.forward(residual, x, add=step.take_owed(residual))
             self.ffn.forward(x, step, residual)

@@ -5,12 +5,14 @@ from __future__ import annotations
 import torch
 
 from kvforge_amd.kernels import ops
-from kvforge_amd.parts.base import FeedForward, WeightSpec
+from kvforge_amd.parts.base import FeedForward, WeightSpec, add_product
 from kvforge_amd.registry import register_feed_forward
 
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    settles_residual = True  # its norm kernel adds what is owed to the stream
+
     def __init__(self, prefix: str, hidden: int, intermediate: int) -> None:
         self.prefix, self.hidden, self.inter = prefix, int(hidden), int(intermediate)
         self.w_gate_up: torch.Tensor | None = None
@@ -57,10 +59,13 @@ class SwiGLU(FeedForward):
         ws, dt, rms = step.ws, step.act_dtype, self.norm_eps
         act = ws.buf("ffn_act", (n, self.inter), dt)
         if rms is not None and not ops.bf16_kernel_takes(x, self.w_gate_up, True):
-            # too many rows for the norm to ride in the projection: a norm kernel of its own
+            # too many rows for the norm to ride in the projection: a norm kernel of its own,
+            # which also adds what the mixer still owes the stream
             normed = ws.buf("normed", (n, self.hidden), dt)
-            ops.rmsnorm(x, None, rms, normed)
+            ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
+        else:
+            step.settle()
         if ops.bf16_kernel_takes(x, self.w_gate_up, rms is not None) and self.inter % 2 == 0:
             # one kernel: (norm,) gate/up projection, SwiGLU gate
             ops.gemm_fused(x, self.w_gate_up, act, rms_eps=rms, silu_pairs=True)
@@ -68,4 +73,4 @@ class SwiGLU(FeedForward):
             gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
             ops.gemm(x, self.w_gate_up, gu)
             ops.silu_mul(gu, act, paired=True)
-        ops.gemm(act, self.w_down, residual, accumulate=True)
+        add_product(step, act, self.w_down, residual)

@@ -29,8 +29,9 @@ class RMSNorm(Norm):
     def num_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
-        ops.rmsnorm(x, self.weight, self.eps, out, rows)
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None,
+                add: torch.Tensor | None = None) -> None:
+        ops.rmsnorm(x, self.weight, self.eps, out, rows, add)
 
     def foldable_into(self, matrix: torch.Tensor) -> bool:
         """Whether this norm's weight may be multiplied into the columns of a bf16 matrix: only

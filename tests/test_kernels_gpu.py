@@ -41,7 +41,34 @@ def test_embed(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("h", [96, 100, 2048, 3000])
+@pytest.mark.parametrize("h", [96, 100, 2048, 5000])
+def test_rmsnorm_with_owed_sum(dtype, h):
+    """norm(x + add): without rows the sum is left in x; with rows x stays as it was."""
+    g = torch.Generator().manual_seed(h + 1)
+    x = torch.randn(7, h, generator=g) * 2
+    add = torch.randn(7, h, generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(h, generator=g)).to(dtype)
+    total = x + add.float()
+    xd = x.to(DEV)
+    out = torch.empty(7, h, dtype=dtype, device=DEV)
+    ops().rmsnorm(xd, w.to(DEV), 1e-5, out, None, add.to(DEV))
+    torch.testing.assert_close(out.float().cpu(), plain.rms_norm(total, w.float(), 1e-5), **tol(dtype))
+    torch.testing.assert_close(xd.cpu(), total, atol=1e-6, rtol=1e-6)
+    rows = torch.tensor([6, 2, 2], dtype=torch.int32)
+    xd = x.to(DEV)
+    out = torch.empty(3, h, dtype=dtype, device=DEV)
+    ops().rmsnorm(xd, None, 1e-5, out, rows.to(DEV), add.to(DEV))
+    want = plain.rms_norm(total[rows.long()], torch.ones(h), 1e-5)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    assert torch.equal(xd.cpu(), x)
+    # the sum alone
+    xd = x.to(DEV)
+    ops().add_rows(xd, add.to(DEV))
+    torch.testing.assert_close(xd.cpu(), total, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h", [96, 100, 2048, 3000, 5000])
 @pytest.mark.parametrize("w32", [False, True])
 def test_rmsnorm(dtype, h, w32):
     g = torch.Generator().manual_seed(h)

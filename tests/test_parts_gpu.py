@@ -83,6 +83,7 @@ def test_swiglu_part(dtype):
     step.ws, step.act_dtype = Workspace(DEV), dtype
     residual = res.clone().to(DEV)
     part.forward(x.to(DEV), step, residual)
+    step.settle()
     want = res + plain.swiglu(x.float(), *(w[f"m.{n}_proj.weight"] for n in ("gate", "up", "down")))
     torch.testing.assert_close(residual.cpu(), want, **tol(dtype))
 
@@ -146,6 +147,7 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
         x = torch.cat([xs[rid][a:b] for rid, a, b in portions]).to(DEV)
         residual = torch.zeros(x.shape[0], hidden, device=DEV)
         part.forward(x, step, ls, residual)
+        step.settle()  # with many rows the last product is left owed to the stream
         off = 0
         for rid, a, b in portions:
             got[rid].append(residual[off:off + b - a].cpu())
@@ -156,7 +158,8 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_pre_norm_block(dtype):
+@pytest.mark.parametrize("n", [7, 23])  # few rows: sums in the product kernels; many: owed to the stream
+def test_pre_norm_block(dtype, n):
     hidden, H, KV, d, inter = 32, 2, 1, 16, 48
     rot = RotaryPositions(d, 100.0)
     rot.prepare(32, DEV)
@@ -168,17 +171,18 @@ def test_pre_norm_block(dtype):
         t = torch.randn(spec.shape, generator=g) * (0.1 if spec.init == "norm" else 0.15)
         w[name] = (t + 1 if spec.init == "norm" else t).to(dtype)
     block.load({k: v.to(DEV) for k, v in w.items()})
-    x = rand(7, hidden, seed=21)
+    x = rand(n, hidden, seed=21)
     cache = CacheManager(4, [CacheGroup((0,), KV, d, None)], 8)
-    cache.allocate("r", 7)
+    cache.allocate("r", n)
     ls = LayerState(group=0, owns_cache=True, k_pages=torch.zeros(8, KV, 4, d, dtype=dtype, device=DEV),
                     v_pages=torch.zeros(8, KV, d, 4, dtype=dtype, device=DEV))
-    step = make_step([StepEntry("r", [0] * 7, 0, "none")], cache, dtype)
+    step = make_step([StepEntry("r", [0] * n, 0, "none")], cache, dtype)
     residual = x.clone().to(DEV)
     block.forward(residual, step, ls)
+    step.settle()
     wf = {k: v.float() for k, v in w.items()}
     cfg = {"num_attention_heads": H, "num_key_value_heads": KV, "head_dim": d}
-    cos, sin = plain.rope_cos_sin(torch.arange(7), plain.rope_inv_freq(d, 100.0))
+    cos, sin = plain.rope_cos_sin(torch.arange(n), plain.rope_inv_freq(d, 100.0))
     h = x + plain.attention_block(plain.rms_norm(x, wf["b.n1.weight"], 1e-5), wf, "b.att.", cfg,
                                   cos, sin, None)
     h = h + plain.swiglu(plain.rms_norm(h, wf["b.n2.weight"], 1e-5), wf["b.ff.gate_proj.weight"],
