@@ -33,7 +33,7 @@ BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
 
 
-def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True):
+def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True, run_steps=None):
     import kvforge_amd
     from kvforge_amd import CacheConfig, EngineConfig, InferenceEngine, SchedulerConfig
 
@@ -43,6 +43,8 @@ def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True
         scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=PREFILL_TOKENS,
                                   max_model_len=CONTEXT_CAP),
         dtype=dtype, use_graphs=use_graphs)
+    if run_steps is not None:
+        cfg.decode_run_steps = run_steps
     return InferenceEngine.from_folder(folder, cfg)
 
 
@@ -62,14 +64,24 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
         engine.add_request(p, params)
     while any(r.is_prefill for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
         engine.step()
-    for _ in range(warmup):
-        engine.step()
+    run_limit = engine.config.decode_run_steps
+
+    def decode_steps(n):
+        """Exactly ``n`` decode steps of the whole batch (the engine may take several between two
+        looks of the host; the last run is cut to fit); returns the tokens produced."""
+        produced, start = 0, engine.runner.num_forward_passes
+        while engine.runner.num_forward_passes - start < n:
+            engine.config.decode_run_steps = min(run_limit, n - (engine.runner.num_forward_passes - start))
+            produced += sum(len(o.new_token_ids) for o in engine.step())
+        engine.config.decode_run_steps = run_limit
+        assert engine.runner.num_forward_passes - start == n
+        return produced
+
+    decode_steps(warmup)
     ctx_start = [r.num_tokens for r in engine.scheduler.running]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    produced = 0
-    for _ in range(steps):
-        produced += sum(len(o.new_token_ids) for o in engine.step())
+    produced = decode_steps(steps)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx_end = [r.num_tokens for r in engine.scheduler.running]
@@ -117,6 +129,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--decode-run-steps", type=int, default=None,
+                    help="decode steps the device takes between two looks of the host (engine default: 8)")
     ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill")
     args = ap.parse_args()
@@ -144,7 +158,7 @@ def main() -> int:
         for b in batches:
             need = b * (args.prompt_len + args.steps + args.warmup + 16)
             engine = build_engine(folder, args.dtype, max(b, 1), max(need, PREFILL_TOKENS + 64),
-                                  use_graphs=not args.no_graphs)
+                                  use_graphs=not args.no_graphs, run_steps=args.decode_run_steps)
             if args.phase != "prefill":
                 results[b] = decode_run(engine, vocab, b, args.prompt_len, args.steps, args.warmup)
             if b == args.batch:
@@ -160,6 +174,7 @@ def main() -> int:
         print(json.dumps({"phase": args.phase, "batch": args.batch, "dtype": args.dtype, **part}))
         return 0
     main_run = results[args.batch]
+    run_steps_used = args.decode_run_steps or kvforge_amd.EngineConfig().decode_run_steps
     step_s = main_run["seconds"] / args.steps
     kv_bytes = args.batch * main_run["mean_ctx"] * nums["kv_values_per_token"] * elem
     achieved = (weight_bytes + kv_bytes) / step_s / 1e9
@@ -181,7 +196,7 @@ def main() -> int:
             "rope": "theta 5e5, llama3 factor 32", "rms_norm_eps": cfg["rms_norm_eps"],
             "global_batch": args.batch, "seq_len": args.prompt_len, "new_tokens": args.steps + 1,
             "context_len": CONTEXT_CAP, "block_size": BLOCK_SIZE, "parallelism": "single-gpu",
-            "sampling": "greedy",
+            "sampling": "greedy", "decode_run_steps": run_steps_used,
         },
         "prefill": {"value": round(n / prefill_s, 1), "tokens": n, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / MFMA_PEAK[args.dtype], 4)},

@@ -178,6 +178,13 @@ class CacheManager:
                 return False
         return True
 
+    def can_append_all(self, wanted: "list[tuple[str, int]]") -> bool:
+        """Room to grow every ``(request_id, total_tokens)`` of ``wanted`` at once."""
+        for g, p in enumerate(self.pools):
+            if sum(self._new_blocks(g, rid, total) for rid, total in wanted) > p.num_free:
+                return False
+        return True
+
     def append_slots(self, request_id: str, total_tokens: int, write_start: int) -> None:
         """Back every position in ``[write_start, total_tokens)`` (and what those queries still
         see) with pages.  All-or-nothing: raises before taking anything if a pool is short."""

@@ -71,9 +71,15 @@ class EngineConfig:
     seed: int = 0
     # Replay pure-decode steps from captured HIP graphs (fixed-address metadata buffers).
     use_graphs: bool = True
+    # When every running request decodes and none waits, the device takes up to this many decode
+    # steps by itself (each sampled token becomes the next input there) before the host reads
+    # the tokens and looks at stop conditions; 1 makes the host look after every step.
+    decode_run_steps: int = 8
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)
+        if self.decode_run_steps < 1:
+            raise ValueError("decode_run_steps must be at least 1")
         # The cache holds what the model computes with (src/tokenvault/config.py:150-151).
         self.cache.dtype = self.dtype
 

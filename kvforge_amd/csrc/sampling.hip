@@ -43,6 +43,7 @@ __device__ __forceinline__ float block_reduce_max(float v, float* sh) {
 __global__ __launch_bounds__(THREADS) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ u,
+    const int* __restrict__ u_step, int u_stride,
     int* __restrict__ tokens) {
   __shared__ float sh[NWAVES];
   __shared__ float seg_sum[NWAVES];
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
     if (w < wave) before += seg_sum[w];
     total += seg_sum[w];
   }
-  const float target = u[row] * total;
+  const float target = u[(u_step ? *u_step * u_stride : 0) + row] * total;
   // the wave whose segment holds the target walks it; the last wave with mass catches overshoot
   const bool mine = part > 0.f && target >= before && (target < before + part);
   if (mine) {
@@ -212,12 +213,47 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
 }
 }  // namespace
 
+// u_step (may be null): a device counter; row r then draws with u[*u_step * u_stride + r], so
+// that a captured launch can be replayed for several decode steps, each with numbers of its own.
 KVF_EXPORT int kvf_sample(const float* logits, int ld, int rows, int V, const float* temperature,
-                          const int* top_k, const float* top_p, const float* u, int* tokens,
-                          hipStream_t s) {
+                          const int* top_k, const float* top_p, const float* u, const int* u_step,
+                          int u_stride, int* tokens, hipStream_t s) {
   if (rows <= 0) return 0;
   if (V <= 0 || ld < V) return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(THREADS), 0, s, logits, ld, V, temperature,
-                     top_k, top_p, u, tokens);
+                     top_k, top_p, u, u_step, u_stride, tokens);
+  return kvf_last_error();
+}
+
+namespace {
+// After a decode step of single tokens: the sampled token of every live sequence (context length
+// above zero; padding sequences stay empty) becomes its next input, one position on, and is
+// kept in row *counter of `ring` for the host, which reads all rows of a run of steps at once.
+__global__ void decode_advance_kernel(const int* __restrict__ sampled, int* __restrict__ token_ids,
+                                      int* __restrict__ positions, int* __restrict__ ctx_lens,
+                                      int* __restrict__ ring, int* __restrict__ counter, int rows,
+                                      int ring_stride, int ring_rows) {
+  const int j = *counter;
+  __syncthreads();  // every thread has read the counter before it moves
+  for (int i = threadIdx.x; i < rows; i += blockDim.x) {
+    const int t = sampled[i];
+    if (j >= 0 && j < ring_rows) ring[j * ring_stride + i] = t;
+    if (ctx_lens[i] > 0) {
+      token_ids[i] = t;
+      positions[i] += 1;
+      ctx_lens[i] += 1;
+    }
+  }
+  if (threadIdx.x == 0) *counter = j + 1;
+}
+}  // namespace
+
+KVF_EXPORT int kvf_decode_advance(const int* sampled, int* token_ids, int* positions, int* ctx_lens,
+                                  int* ring, int* counter, int rows, int ring_stride, int ring_rows,
+                                  hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (rows > ring_stride || ring_rows <= 0) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(decode_advance_kernel, dim3(1), dim3(256), 0, s, sampled, token_ids, positions,
+                     ctx_lens, ring, counter, rows, ring_stride, ring_rows);
   return kvf_last_error();
 }

@@ -227,13 +227,16 @@ class Step:
 
 def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], tables_of, slot_of,
               block_size: int, pad_to: int | None = None,
-              windowed_groups: Sequence[bool] | None = None, serial_of=None) -> list[int]:
+              windowed_groups: Sequence[bool] | None = None, serial_of=None,
+              lookahead: int = 0) -> list[int]:
     """Write the batch into ``meta`` (one host-to-device copy) and point ``step`` at it.
     ``tables_of(request_id, group) -> list[int]``; ``slot_of(request_id) -> int``.
     ``pad_to``: pad a pure-decode batch with empty sequences up to this many.
     ``windowed_groups[g]``: group ``g`` gives pages back while a request lives, so its rows are
     rewritten whole every step.  ``serial_of(request_id)`` tells a request id that was freed and
     allocated again from its former self (without it rows are always rewritten whole).
+    ``lookahead``: the tables also carry the pages of this many positions past the step's, for
+    further decode steps that the device advances to by itself.
     Returns how many logits rows each entry gets."""
     B = len(entries)
     q_lens = [len(e.token_ids) for e in entries]
@@ -295,7 +298,7 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
         windowed = windowed_groups is not None and windowed_groups[g]
         for b, e in enumerate(entries):
             t = tables_of(e.request_id, g)
-            need = -(-int(ctx[b]) // block_size)
+            need = -(-(int(ctx[b]) + lookahead) // block_size)
             if need > w or need > len(t):
                 raise ValueError(f"request {e.request_id} needs {need} pages in group {g}; "
                                  f"table holds {len(t)}, width {w}")

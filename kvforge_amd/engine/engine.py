@@ -125,14 +125,53 @@ class InferenceEngine:
         sched = self.scheduler.schedule()
         if sched.is_empty:
             return []
-        new_tokens = self._run(sched.scheduled)
+        run = self._decode_run_length(sched)
+        new_tokens = self._run(sched.scheduled, run)
         outputs = self._postprocess(sched.scheduled, new_tokens)
-        self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens,
+        self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens * run,
                                  time.perf_counter() - t0,
                                  1.0 - self.cache.num_free_blocks / max(1, self.cache.num_blocks))
         return outputs
 
-    def _run(self, group: list[ScheduledRequest]) -> dict[str, int]:
+    def _decode_run_length(self, sched) -> int:
+        """How many decode steps the device takes before the host looks again: more than one
+        only while every scheduled request decodes, nobody waits for admission, no request can
+        reach its length limit inside the run, and the pages of the run's positions are free."""
+        limit = self.config.decode_run_steps
+        group = sched.scheduled
+        if (limit <= 1 or sched.preempted or self.scheduler.num_waiting
+                or any(s.is_prefill or s.num_new_tokens != 1 for s in group)):
+            return 1
+        max_len = self.config.scheduler.max_model_len
+        for s in group:
+            r = s.request
+            limit = min(limit, r.sampling_params.max_tokens - r.num_output_tokens,
+                        max_len - r.num_tokens)
+        if limit <= 1:
+            return 1
+        entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
+                   for s in group]
+        if not self.runner.graph_takes(entries, len(entries)):
+            return 1
+        wanted = [(s.request.request_id, s.request.num_computed_tokens + limit) for s in group]
+        if not self.cache.can_append_all(wanted):
+            return 1
+        for s, (rid, total) in zip(group, wanted):
+            self.cache.append_slots(rid, total, s.request.num_computed_tokens)
+        return limit
+
+    def _run(self, group: list[ScheduledRequest], run: int = 1) -> dict[str, list[int]]:
+        if run > 1:
+            reqs = [s.request for s in group]
+            entries = [StepEntry(r.request_id, r.token_slice(r.num_computed_tokens, 1),
+                                 r.num_computed_tokens, "last") for r in reqs]
+            steps = self.runner.decode_run(entries, self.sampler.seed,
+                                           [r.sampling_params for r in reqs],
+                                           [r.sample_stream for r in reqs],
+                                           [r.num_output_tokens for r in reqs], run)
+            for r in reqs:
+                r.num_computed_tokens += 1
+            return {r.request_id: [step[i] for step in steps] for i, r in enumerate(reqs)}
         entries: list[StepEntry] = []
         sampled: list[Request] = []
         for s in group:
@@ -149,9 +188,9 @@ class InferenceEngine:
                                              [r.num_output_tokens for r in sampled])
         for s in group:
             s.request.num_computed_tokens += s.num_new_tokens
-        return {r.request_id: t for r, t in zip(sampled, tokens)}
+        return {r.request_id: [t] for r, t in zip(sampled, tokens)}
 
-    def _postprocess(self, scheduled: list[ScheduledRequest], new_tokens: dict[str, int]
+    def _postprocess(self, scheduled: list[ScheduledRequest], new_tokens: dict[str, list[int]]
                      ) -> list[RequestOutput]:
         now = time.perf_counter()
         max_len = self.config.scheduler.max_model_len
@@ -160,11 +199,14 @@ class InferenceEngine:
             r = s.request
             emitted: list[int] = []
             reason: FinishReason | None = None
-            if r.request_id in new_tokens:
-                t = new_tokens[r.request_id]
+            for j, t in enumerate(new_tokens.get(r.request_id, ())):
+                if j > 0:
+                    r.num_computed_tokens += 1  # the step that took the token before as its input
                 r.append_token(t, now)
                 emitted.append(t)
                 reason = r.check_stop(max_len)
+                if reason is not None:
+                    break  # what the device sampled past a stop is dropped
             if reason is not None:
                 self.scheduler.finish_request(r, reason)
                 self.metrics.record_finished(r)

@@ -58,9 +58,14 @@ class ModelRunner:
         self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
         self.num_graph_replays = 0
         cap = self.meta.max_seqs
-        self._sample_f = torch.zeros(3 * cap, dtype=torch.float32, device=self.device)
+        # floats: temperatures, top-p, then MAX_DECODE_RUN rows of uniform numbers; ints: top-k,
+        # the sampled tokens, then the counter of steps in a run and the ring of their tokens
+        nf = (2 + MAX_DECODE_RUN) * cap
+        self._sample_f = torch.zeros(nf, dtype=torch.float32, device=self.device)
         self._sample_i = torch.zeros(2 * cap, dtype=torch.int32, device=self.device)
-        self._sample_f_host = torch.zeros(3 * cap, dtype=torch.float32, pin_memory=True)
+        self._run_counter = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self._run_ring = torch.zeros(MAX_DECODE_RUN, cap, dtype=torch.int32, device=self.device)
+        self._sample_f_host = torch.zeros(nf, dtype=torch.float32, pin_memory=True)
         self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
         self._sample_f_np, self._sample_i_np = self._sample_f_host.numpy(), self._sample_i_host.numpy()
         self._sample_ids: list[str] = []
@@ -74,16 +79,16 @@ class ModelRunner:
     def _slot_of(self, request_id: str) -> int:
         return self.cache.slots.slot(request_id) if self.cache.slots.num_slots else -1
 
-    def build_step(self, entries: Sequence[StepEntry], pad_to: int | None = None
-                   ) -> tuple[Step, list[int]]:
+    def build_step(self, entries: Sequence[StepEntry], pad_to: int | None = None,
+                   lookahead: int = 0) -> tuple[Step, list[int]]:
         for e in entries:
-            if e.start_pos + len(e.token_ids) > self.max_model_len:
+            if e.start_pos + len(e.token_ids) + lookahead > self.max_model_len:
                 raise ValueError(f"request {e.request_id} would pass max_model_len "
                                  f"{self.max_model_len}")
         step = Step()
         step.ws, step.act_dtype, step.device = self.ws, self.model.dtype, self.device
         counts = fill_step(step, self.meta, entries, self.cache.block_table, self._slot_of,
-                           self.block_size, pad_to, self._windowed, self.cache.serial)
+                           self.block_size, pad_to, self._windowed, self.cache.serial, lookahead)
         return step, counts
 
     @torch.inference_mode()
@@ -96,30 +101,47 @@ class ModelRunner:
         self.num_tokens_processed += step.n_tokens
         return logits
 
+    def graph_takes(self, entries: Sequence[StepEntry], num_params: int) -> bool:
+        """Whether a step goes through the captured decode path: single tokens that each want
+        their logits, within the largest captured batch."""
+        b = len(entries)
+        return (self.use_graphs and b == num_params and b <= GRAPH_MAX_BATCH
+                and all(len(e.token_ids) == 1 and e.want == "last" for e in entries))
+
     @torch.inference_mode()
     def step_and_sample(self, entries: Sequence[StepEntry], sampler, params, streams, counters
                         ) -> list[int]:
         """One forward, then one token for every wanted place (in row order)."""
-        b = len(entries)
-        if (self.use_graphs and b == len(params) and b <= GRAPH_MAX_BATCH
-                and all(len(e.token_ids) == 1 and e.want == "last" for e in entries)):
-            return self._decode_step(entries, sampler.seed, params, streams, counters)
+        if self.graph_takes(entries, len(params)):
+            return self.decode_run(entries, sampler.seed, params, streams, counters, 1)[0]
         logits = self.step(entries)
         if logits.shape[0] != len(params):
             raise ValueError("one SamplingParams per wanted place")
         return sampler(logits, params, streams, counters)
 
     # ------------------------------------------------------------------ decode through graphs
-    def _decode_step(self, entries, seed, params, streams, counters) -> list[int]:
-        """A step of single tokens, padded to a bucket of batch sizes so that its launches can be
-        captured once in a HIP graph and replayed: metadata and sampling parameters live at fixed
-        device addresses and are refreshed by two copies before each replay."""
+    @torch.inference_mode()
+    def decode_run(self, entries, seed, params, streams, counters, num_steps: int = 1
+                   ) -> list[list[int]]:
+        """``num_steps`` decode steps of single tokens with one wait for the device at the end;
+        returns the tokens of every step, ``[step][entry]``.
+
+        The batch is padded to a bucket of sizes so that its launches are captured once in a HIP
+        graph and replayed: metadata and sampling parameters live at fixed device addresses and
+        are refreshed by two copies before the run.  The graph ends with a kernel that turns each
+        sampled token into the sequence's next input, so further steps need nothing from the
+        host; the pages of their positions must be in the requests' tables already."""
         b = len(entries)
+        k = int(num_steps)
+        if not 1 <= k <= MAX_DECODE_RUN:
+            raise ValueError(f"a run holds 1 to {MAX_DECODE_RUN} steps")
+        if not self.graph_takes(entries, len(params)):
+            raise ValueError("a decode run takes single tokens that each want their logits")
         bucket = 1
         while bucket < b:
             bucket *= 2
         bucket = min(bucket, self.meta.max_seqs)
-        step, _ = self.build_step(entries, pad_to=bucket)
+        step, _ = self.build_step(entries, pad_to=bucket, lookahead=k - 1)
         # The longest context enters the captured launches only through the number of cuts of
         # the key range, which grows by one per DECODE_KEYS_PER_SPLIT keys up to a limit: graphs
         # are kept per such cell, planned for the cell's lower edge.
@@ -132,7 +154,7 @@ class ModelRunner:
             # the batch changed: rewrite the per-row parameters (padding rows are greedy)
             fh[:bucket] = 0.0
             fh[cap:cap + bucket] = 1.0
-            fh[2 * cap:2 * cap + bucket] = 0.0
+            fh[2 * cap:] = 0.0
             ih[:bucket] = 0
             for i, p in enumerate(params):
                 fh[i], fh[cap + i], ih[i] = p.temperature, p.top_p, p.top_k
@@ -143,29 +165,35 @@ class ModelRunner:
         else:
             dirty = bool(self._sample_drawn)
         for i in self._sample_drawn:
-            fh[2 * cap + i] = uniform(seed, streams[i], counters[i])
+            for j in range(k):
+                fh[(2 + j) * cap + i] = uniform(seed, streams[i], counters[i] + j)
         if dirty:
             self._sample_f.copy_(self._sample_f_host, non_blocking=True)
+        self._run_counter.zero_()
         key = (bucket, ctx_bucket)
         graph = self.graphs.get(key)
+        replays = k
         if graph is None:
-            self._forward_and_sample(step, bucket)          # the real result, and a warm-up
-            tokens = self._sample_i[cap:cap + b].tolist()
-            self.graphs[key] = self._capture(step, bucket)
-        else:
+            self._forward_and_sample(step, bucket)          # the first step, and a warm-up
+            graph = self.graphs[key] = self._capture(step, bucket)
+            replays -= 1
+        for _ in range(replays):
             graph.graph.replay()
-            self.num_graph_replays += 1
-            tokens = self._sample_i[cap:cap + b].tolist()
-        self.num_forward_passes += 1
-        self.num_tokens_processed += b
+        self.num_graph_replays += replays
+        tokens = self._run_ring[:k, :b].tolist()
+        self.num_forward_passes += k
+        self.num_tokens_processed += b * k
         return tokens
 
     def _forward_and_sample(self, step: Step, rows: int) -> torch.Tensor:
         cap = self.meta.max_seqs
         logits = self.model.forward(step)
+        sampled = self._sample_i[cap:cap + rows]
         ops.sample(logits, self._sample_f[:rows], self._sample_i[:rows],
-                   self._sample_f[cap:cap + rows], self._sample_f[2 * cap:2 * cap + rows],
-                   self._sample_i[cap:cap + rows])
+                   self._sample_f[cap:cap + rows], self._sample_f[2 * cap:].view(MAX_DECODE_RUN, cap),
+                   sampled, self._run_counter)
+        ops.decode_advance(sampled, step.token_ids, step.positions, step.ctx_lens, self._run_ring,
+                           self._run_counter)
         return logits
 
     def _capture(self, step: Step, rows: int) -> "_DecodeGraph":
@@ -182,6 +210,7 @@ class ModelRunner:
 
 
 GRAPH_MAX_BATCH = 128  # beyond this the matrix products leave the weight-streaming kernel
+MAX_DECODE_RUN = 16    # decode steps the device can take by itself before the host looks
 
 
 class _DecodeGraph:

@@ -48,6 +48,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     p.add_argument("--max-num-batched-tokens", type=int, default=2048)
     p.add_argument("--max-model-len", type=int, default=2048)
     p.add_argument("--no-graphs", action="store_true", help="do not replay decode steps from HIP graphs")
+    p.add_argument("--decode-run-steps", type=int, default=8,
+                   help="decode steps the device takes between two looks of the host")
     p.add_argument("--json", action="store_true", help="print one JSON object instead of text")
     return p.parse_args(argv)
 
@@ -77,7 +79,8 @@ def main(argv: list[str] | None = None) -> int:
         scheduler=SchedulerConfig(max_num_seqs=args.max_num_seqs,
                                   max_num_batched_tokens=args.max_num_batched_tokens,
                                   max_model_len=args.max_model_len),
-        device=args.device, dtype=args.dtype, seed=args.seed, use_graphs=not args.no_graphs)
+        device=args.device, dtype=args.dtype, seed=args.seed, use_graphs=not args.no_graphs,
+        decode_run_steps=args.decode_run_steps)
     if args.model:
         engine = InferenceEngine.from_folder(args.model, config, tokenizer)
         name = args.model

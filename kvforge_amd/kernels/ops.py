@@ -454,22 +454,54 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
 
 # ------------------------------------------------------------------------------ sampling
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None,
-           top_p: torch.Tensor | None, u: torch.Tensor, tokens: torch.Tensor) -> None:
+           top_p: torch.Tensor | None, u: torch.Tensor, tokens: torch.Tensor,
+           u_step: torch.Tensor | None = None) -> None:
     """One token per row of fp32 ``logits``: argmax where ``temperature == 0``, otherwise the
-    inverse CDF of the processed distribution at ``u``."""
+    inverse CDF of the processed distribution at ``u``.  With ``u_step`` (one int32 on the
+    device) ``u`` holds several rows of numbers, ``[steps, row stride]``, and row ``u_step[0]``
+    is used: a captured launch then serves several decode steps."""
     _check(logits, "logits", F32, (None, None), contiguous=False)
     if logits.stride(1) != 1:
         raise KernelError("sample: logits rows must be dense")
     r, v = logits.shape
     _check(temperature, "temperature", F32, (r,))
-    _check(u, "u", F32, (r,))
+    stride = 0
+    if u_step is None:
+        _check(u, "u", F32, (r,))
+    else:
+        _check(u_step, "u_step", I32, (1,))
+        _check(u, "u", F32, (None, None))
+        stride = u.shape[1]
+        if stride < r:
+            raise KernelError("sample: rows of u are shorter than the batch")
     _check(tokens, "tokens", I32, (r,))
     if top_k is not None:
         _check(top_k, "top_k", I32, (r,))
     if top_p is not None:
         _check(top_p, "top_p", F32, (r,))
-    f = _fn("sampling", "kvf_sample", [c_void_p, c_int, c_int, c_int] + [c_void_p] * 6)
+    f = _fn("sampling", "kvf_sample",
+            [c_void_p, c_int, c_int, c_int] + [c_void_p] * 5 + [c_int, c_void_p, c_void_p])
     _ok(f(logits.data_ptr(), logits.stride(0) if r > 1 else v, r, v, temperature.data_ptr(),
           top_k.data_ptr() if top_k is not None else None,
-          top_p.data_ptr() if top_p is not None else None, u.data_ptr(), tokens.data_ptr(),
+          top_p.data_ptr() if top_p is not None else None, u.data_ptr(),
+          u_step.data_ptr() if u_step is not None else None, stride, tokens.data_ptr(),
           _stream()), "sample")
+
+
+def decode_advance(sampled: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
+                   ctx_lens: torch.Tensor, ring: torch.Tensor, counter: torch.Tensor) -> None:
+    """After a step of single tokens: ``ring[counter[0]] = sampled``; for every sequence with a
+    context, the sampled token becomes the next input (``token_ids``), ``positions`` and
+    ``ctx_lens`` move on by one; ``counter[0] += 1``.  All on the device, in stream order."""
+    r = sampled.shape[0]
+    for t, name in ((sampled, "sampled"), (token_ids, "token_ids"), (positions, "positions"),
+                    (ctx_lens, "ctx_lens")):
+        _check(t, name, I32, (r,))
+    _check(ring, "ring", I32, (None, None))
+    _check(counter, "counter", I32, (1,))
+    if ring.shape[1] < r:
+        raise KernelError("decode_advance: rows of the ring are shorter than the batch")
+    f = _fn("sampling", "kvf_decode_advance", [c_void_p] * 6 + [c_int] * 3 + [c_void_p])
+    _ok(f(sampled.data_ptr(), token_ids.data_ptr(), positions.data_ptr(), ctx_lens.data_ptr(),
+          ring.data_ptr(), counter.data_ptr(), r, ring.shape[1], ring.shape[0], _stream()),
+        "decode_advance")

@@ -140,7 +140,7 @@ def test_batched_output_equals_isolated_greedy(model_a, dtype):
 def test_requests_join_running_batch(model_a):
     folder, oracle = model_a
     prompts = prompts_for(256, 4, 1)
-    engine = engine_for(folder)
+    engine = engine_for(folder, decode_run_steps=1)   # the test counts steps of one token
     engine.add_request(prompts[0], GREEDY, request_id="r0")
     engine.add_request(prompts[1], GREEDY, request_id="r1")
     done, step = {}, 0
@@ -249,6 +249,41 @@ def test_sampling_does_not_depend_on_batching(model_b):
     assert again == alone and other_seed != alone
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_runs_of_decode_steps_on_the_device_equal_single_steps(model_b, dtype):
+    """With nothing waiting the device takes several decode steps before the host looks (each
+    sampled token becomes the next input there).  Tokens, stop handling, lengths that are no
+    multiple of the run, pages that begin inside a run and freed pages must all be what single
+    steps give, for greedy and for drawn tokens."""
+    folder, oracle = model_b
+    prompts = prompts_for(384, 4, 21, 3, 40)
+    params = [SamplingParams(max_tokens=21, temperature=0.0),
+              SamplingParams(max_tokens=13, temperature=0.9, top_k=40, top_p=0.95, seed=3),
+              SamplingParams(max_tokens=30, temperature=0.0),
+              SamplingParams(max_tokens=5, temperature=1.0, seed=4)]
+    single = engine_for(folder, dtype, decode_run_steps=1, seed=2)
+    want = single.generate(prompts, params)
+    for run in (2, 8, 16):
+        engine = engine_for(folder, dtype, decode_run_steps=run, seed=2)
+        got = engine.generate(prompts, params)
+        for g, w in zip(got, want):
+            assert g.output_token_ids == w.output_token_ids and g.finish_reason == w.finish_reason
+        assert engine.runner.num_forward_passes < single.runner.num_forward_passes + 4 * run
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+    if dtype == "float32":
+        oracle.check_choices(prompts[0], want[0].output_token_ids, 1e-4)
+        oracle.check_choices(prompts[2], want[2].output_token_ids, 1e-4)
+    # a stop token inside a run: what the device sampled after it is dropped
+    stop = want[2].output_token_ids[10]
+    first = want[2].output_token_ids.index(stop)
+    engine = engine_for(folder, dtype, decode_run_steps=8, seed=2)
+    out = engine.generate([prompts[2]], SamplingParams(max_tokens=30, temperature=0.0,
+                                                      stop_token_ids=[stop]))[0]
+    assert out.output_token_ids == want[2].output_token_ids[:first + 1]
+    assert out.finish_reason == "stop"
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
 def test_rejections_at_the_entry_point(model_a):
     folder, _ = model_a
     engine = engine_for(folder)
@@ -306,8 +341,10 @@ def test_graph_replay_equals_eager_steps(model_b, dtype):
                                  (45, 1.2, 10, 1.0))]
 
     def run(use_graphs):
+        # one token per step in both runs: the same steps then hold the same requests, and bf16
+        # logits (hence drawn tokens) are compared bit for bit
         engine = engine_for(folder, dtype, block_size=8, max_num_seqs=5, max_num_batched_tokens=32,
-                            seed=11, use_graphs=use_graphs)
+                            seed=11, use_graphs=use_graphs, decode_run_steps=1)
         done, step = {}, 0
         pending = list(zip(prompts, params))
         for p, sp in pending[:3]:
