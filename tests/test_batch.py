@@ -75,6 +75,24 @@ def test_pure_decode_padding_is_inert():
                   pad_to=2)
 
 
+def test_tables_carry_the_pages_of_a_run_of_decode_steps():
+    """``lookahead``: the tables hold the pages of positions the device will reach by itself,
+    and a table that lacks them is refused; what is owed to the stream is settled on demand."""
+    cache, meta, step = setup()
+    cache.allocate("a", 4)                      # one page of 4 tokens, full
+    with pytest.raises(ValueError, match="pages"):
+        fill_step(step, meta, [StepEntry("a", [7], 3, "last")], cache.block_table, lambda r: -1, 4,
+                  pad_to=2, lookahead=3)
+    assert cache.can_append_all([("a", 7)])
+    cache.append_slots("a", 7, 3)               # positions 4..6 of the run
+    fill_step(step, meta, [StepEntry("a", [7], 3, "last")], cache.block_table, lambda r: -1, 4,
+              pad_to=2, lookahead=3)
+    assert step.block_tables[0][0, :2].tolist() == cache.block_table("a")
+    assert step.ctx_lens.tolist() == [4, 0]
+    assert not cache.can_append_all([("a", 4 * 16 + 1)])   # more pages than the pool has
+    assert step.take_owed(torch.zeros(1)) is None
+
+
 def test_refusals():
     cache, meta, step = setup()
     cache.allocate("a", 4)
