@@ -427,14 +427,15 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 
 // ------------------------------------------------------------------------- few rows, split keys
 // TWO: a wave holds the fragments of two blocks, loading one while it consumes the other.
-template <int DT, bool TWO>
-__global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
+// NW: waves of the workgroup; more of them shorten each wave's walk over its cut of the keys.
+template <int DT, bool TWO, int NW>
+__global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
     const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     bf16_t* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_ml, MArgs a) {
   constexpr int DC = (DT + 1) / 2;
-  extern __shared__ float lds[];  // [WAVES][DT][64][4] accumulators, then [WAVES][16][2]
+  extern __shared__ float lds[];  // [NW][DT][64][4] accumulators, then [NW][16][2]
 
   const int lane = threadIdx.x % KVF_WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KVF_WAVE);  // the same in all lanes
@@ -461,10 +462,10 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_ke
   const int kb0 = (lo / 32) * 32;
   const int blocks = hi >= kb0 ? (hi - kb0) / 32 + 1 : 0;
   int per = (blocks + a.splits - 1) / a.splits;
-  per = (per + WAVES - 1) / WAVES * WAVES;  // whole rounds of the four waves
+  per = (per + NW - 1) / NW * NW;  // whole rounds of the waves
   const int kb_end = min(hi + 1, kb0 + (static_cast<int>(blockIdx.z) + 1) * per * 32);
   const int kb_begin = kb0 + (blockIdx.z * per + wave) * 32;
-  constexpr int STEP = 32 * WAVES;
+  constexpr int STEP = 32 * NW;
   const float scale2 = a.scale * LOG2E;
 
   float m_ref[1] = {-INFINITY}, l_run[1] = {0.f};
@@ -532,9 +533,9 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_ke
     }
   }
 
-  // ---- merge the four waves, then store or hand on the partial result
-  float* red_acc = lds;                             // [WAVES][DT][64][4]
-  float* red_ml = lds + WAVES * DT * KVF_WAVE * 4;  // [WAVES][16][2]
+  // ---- merge the waves, then store or hand on the partial result
+  float* red_acc = lds;                             // [NW][DT][64][4]
+  float* red_ml = lds + NW * DT * KVF_WAVE * 4;  // [NW][16][2]
   const float l_row = row_sum(l_run[0]);
 #pragma unroll
   for (int t = 0; t < DT; ++t)
@@ -546,10 +547,10 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_ke
   __syncthreads();
   float mm = -INFINITY;
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) mm = fmaxf(mm, red_ml[(w * 16 + j16) * 2]);
-  float cw[WAVES], ll = 0.f;
+  for (int w = 0; w < NW; ++w) mm = fmaxf(mm, red_ml[(w * 16 + j16) * 2]);
+  float cw[NW], ll = 0.f;
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
+  for (int w = 0; w < NW; ++w) {
     const float mw = red_ml[(w * 16 + j16) * 2];
     cw[w] = mw == -INFINITY ? 0.f : exp2f(mw - mm);
     ll += red_ml[(w * 16 + j16) * 2 + 1] * cw[w];
@@ -562,10 +563,10 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_ke
     part_ml[slot * 2 + 1] = ll;
   }
   const float inv = ll > 0.f ? 1.f / ll : 0.f;
-  for (int t = wave; t < DT; t += WAVES) {  // wave w finishes element tiles w, w + 4, ...
+  for (int t = wave; t < DT; t += NW) {  // wave w finishes element tiles w, w + NW, ...
     f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w)
+    for (int w = 0; w < NW; ++w)
       o += *reinterpret_cast<const f32x4*>(red_acc + ((w * DT + t) * KVF_WAVE + lane) * 4) * cw[w];
     const int e0 = t * 16 + 4 * kg;
     if (a.splits == 1)
@@ -637,15 +638,31 @@ void launch_runs(dim3 grid, hipStream_t s, const void* q, const void* k_pages, c
                      static_cast<bf16_t*>(out), a);
 }
 
+template <int DT, int NW>
+void launch_split_waves(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
+                        const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
+                        void* out, float* part_acc, float* part_ml, const MArgs& a) {
+  const size_t lds = (static_cast<size_t>(NW) * DT * KVF_WAVE * 4 + NW * 16 * 2) * sizeof(float);
+  hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW>), grid, dim3(NW * KVF_WAVE), lds, s,
+                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                     static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                     static_cast<bf16_t*>(out), part_acc, part_ml, a);
+}
+
+// Eight waves shorten each wave's walk over the keys when the grid leaves compute units idle
+// anyway (and two blocks of fragments still fit the registers that leaves each wave); a grid
+// that fills the chip does better with four.
 template <int DT>
 void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
                   const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
                   void* out, float* part_acc, float* part_ml, const MArgs& a) {
-  const size_t lds = (static_cast<size_t>(WAVES) * DT * KVF_WAVE * 4 + WAVES * 16 * 2) * sizeof(float);
-  hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8)>), grid, dim3(256), lds, s,
-                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
-                     static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
-                     static_cast<bf16_t*>(out), part_acc, part_ml, a);
+  const size_t groups = static_cast<size_t>(grid.x) * grid.y * grid.z;
+  if (DT <= 6 && groups <= 256)
+    launch_split_waves<DT, (DT <= 6 ? 8 : 4)>(grid, s, q, k_pages, vt_pages, block_table, seq_ids, cu_q,
+                                              ctx_lens, out, part_acc, part_ml, a);
+  else
+    launch_split_waves<DT, 4>(grid, s, q, k_pages, vt_pages, block_table, seq_ids, cu_q, ctx_lens, out,
+                              part_acc, part_ml, a);
 }
 
 #define KVF_EACH_DT(X) \
