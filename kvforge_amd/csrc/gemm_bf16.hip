@@ -25,6 +25,14 @@
 //   straight into the pages of the token's sequence (K pages [nb, KV, block, d], V pages
 //   transposed [nb, KV, d, block]).
 // K must be a multiple of 8 (16-byte loads); a k-step that passes K loads zeros.
+//
+// Layout of W.  In the checkpoint's row-major [N, K] a wave's load of one operand fragment
+// touches 16 rows, 64 bytes each: 16 cache lines per group of 16 lanes, and the L1 looks lines up
+// one at a time, which bounds the kernel far below what HBM delivers.  The engine therefore also
+// keeps W in tiles (`w_tiled`): [ceil(N/16)][ceil(K/32)][64 lanes][8 elements], tile (g, s) being
+// rows 16g..16g+15, columns 32s..32s+31 in the order the instruction wants them (lane
+// 16*c + r holds row r, columns 8c..8c+7), zero-padded.  A fragment is then 1 KB of consecutive
+// bytes.  Both layouts give the same bits.
 #include "common.h"
 
 namespace {
@@ -203,31 +211,40 @@ constexpr int depth(int mt, int nt, int at) {
   return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : (mt * nt == 1 ? 8 : mt * nt <= 4 ? 4 : 2);
 }
 
-// RW: rows of W one workgroup owns (16, 8 or 4).  With fewer than 16 the instruction's other
-// rows repeat them (same addresses, no extra memory traffic) and are dropped at the store: it
-// trades matrix-core work, which is free here, for more workgroups when N is small.
-template <int MT, int NT, int AT, int EPI, int RW>
+template <int MT, int NT, int AT, int EPI>
 __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
-    int K, int lda, int ldc, int m_base, float eps, RopeEpi rp) {
+    int K, int lda, int ldc, int m_base, float eps, int w_tiled, RopeEpi rp) {
+  constexpr int RW = 16;  // rows of W per group
   extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
   const int nw = blockDim.x / KVF_WAVE;
   const int n0 = blockIdx.x * RW * NT;
   const int r16 = lane % 16, kg = lane / 16;
+  const int ksteps = (K + 31) / 32;
+  // where this lane's fragment of k-step 0 lies, and how far the next k-step is
   const bf16_t* wp[NT];
+  const size_t w_step = w_tiled ? KVF_WAVE * 8 : 32;
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
-    int wrow = n0 + j * RW + r16 % RW;
-    if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
-    wp[j] = W + static_cast<size_t>(wrow) * K + kg * 8;
+    if (w_tiled) {
+      const int group = min(static_cast<int>(blockIdx.x) * NT + j, (N + RW - 1) / RW - 1);
+      wp[j] = W + (static_cast<size_t>(group) * ksteps * KVF_WAVE + lane) * 8;
+    } else {
+      int wrow = n0 + j * RW + r16;
+      if (wrow >= N) wrow = N - 1;  // clamped rows are computed and never stored
+      wp[j] = W + static_cast<size_t>(wrow) * K + kg * 8;
+    }
   }
   size_t aoff[MT];
+  bool a_live[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    int arow = m_base + t * 16 + r16;
-    if (arow >= M) arow = M - 1;  // rows past M repeat the last one and are never stored
-    aoff[t] = static_cast<size_t>(arow) * lda + kg * 8;
+    // Rows past M are not loaded at all (their lanes hold zeros and are never stored): a wave's
+    // load touches one cache line per row it reads, and the L1 looks lines up one at a time.
+    const int arow = m_base + t * 16 + r16;
+    a_live[t] = arow < M;
+    aoff[t] = static_cast<size_t>(a_live[t] ? arow : 0) * lda + kg * 8;
   }
   const bf16_t* Ab = static_cast<const bf16_t*>(Av);
   const float* Af = static_cast<const float*>(Av);
@@ -247,14 +264,13 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 #pragma unroll
   for (int j = 0; j < NT; ++j) pre[j].have = false;
   const int pre_m = m_base + r16, pre_n = n0 + 4 * kg;
-  const bool pre_mine = PRE && wave == 0 && pre_m < M && 4 * kg < RW;
+  const bool pre_mine = PRE && wave == 0 && pre_m < M;
   if (pre_mine) {
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       if (pre_n + j * RW < N) epi_prefetch_a<EPI>(pre[j], pre_m, pre_n + j * RW, N, ldc, Cv, rp);
   }
 
-  const int ksteps = (K + 31) / 32;
   constexpr int U = depth(MT, NT, AT);
   int ks = wave;
   bool first = true;
@@ -265,10 +281,11 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       const int k = (ks + u * nw) * 32;
       const bool ok = k + kg * 8 + 8 <= K;
 #pragma unroll
-      for (int j = 0; j < NT; ++j) wf[u][j] = load_frag(wp[j] + k, ok);
+      for (int j = 0; j < NT; ++j) wf[u][j] = load_frag(wp[j] + (ks + u * nw) * w_step, ok || w_tiled);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        af[u][t] = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
+        af[u][t] = AT ? load_frag_f32(Af + aoff[t] + k, ok && a_live[t], ss[t])
+                      : load_frag(Ab + aoff[t] + k, ok && a_live[t]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -297,10 +314,11 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
     bf16x8 af[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
-      af[t] = AT ? load_frag_f32(Af + aoff[t] + k, ok, ss[t]) : load_frag(Ab + aoff[t] + k, ok);
+      af[t] = AT ? load_frag_f32(Af + aoff[t] + k, ok && a_live[t], ss[t])
+                 : load_frag(Ab + aoff[t] + k, ok && a_live[t]);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const bf16x8 wf = load_frag(wp[j] + k, ok);
+      const bf16x8 wf = load_frag(wp[j] + ks * w_step, ok || w_tiled);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
         acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af[t], acc[j][t], 0, 0, 0);
@@ -331,7 +349,7 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
         s += *reinterpret_cast<const f32x4*>(red + ((w * MT + t) * KVF_WAVE + l) * 4);
       const int m = m_base + t * 16 + l % 16;
       const int n = n0 + j * RW + 4 * (l / 16);
-      if (m >= M || n >= N || 4 * (l / 16) >= RW) continue;
+      if (m >= M || n >= N) continue;
       if (AT) {
         float tot = 0.f;
         for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
@@ -358,16 +376,16 @@ int pick_waves(int K) {
   return nw;
 }
 
-template <int MT, int NT, int AT, int EPI, int RW = 16>
+template <int MT, int NT, int AT, int EPI>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-               int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
-  const int groups = (N + RW * NT - 1) / (RW * NT);
+               int m_base, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
+  const int groups = (N + 16 * NT - 1) / (16 * NT);
   int nw = pick_waves(K);
   if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
   const dim3 grid(groups), block(nw * KVF_WAVE);
   const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, RW>), grid, block, lds, s, A, W, C, M, N, K,
-                     lda, ldc, m_base, eps, rp);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
+                     lda, ldc, m_base, eps, w_tiled, rp);
   return kvf_last_error();
 }
 
@@ -375,49 +393,47 @@ int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int
 // spare (the grid must still fill the chip).
 template <int MT, int AT, int EPI>
 int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-              int m_base, float eps, const RopeEpi& rp, hipStream_t s) {
+              int m_base, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
   const int tiles = (N + 15) / 16;
   if (MT >= 2 && MT <= 4 && !AT) {
     if (MT == 4 && tiles >= 1024)
-      return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+      return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
     if (tiles >= 512)
-      return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+      return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
   }
   if (MT == 1) {
     // Every workgroup reads all of A, so with several rows of A and many rows of W a workgroup
-    // takes 32 rows of W and halves that traffic; fewer than 16 rows measured no gain anywhere.
+    // takes 32 rows of W and halves that traffic.
     const int rw = g_rows_override > 0 ? g_rows_override : (M - m_base > 4 && tiles >= 512 ? 32 : 16);
-    if (rw == 4) return launch_one<1, 1, AT, EPI, 4>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    if (rw == 8) return launch_one<1, 1, AT, EPI, 8>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
   }
-  return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+  return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
 }
 
 template <int AT, int EPI>
 int launch_rows(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-                float eps, const RopeEpi& rp, hipStream_t s) {
+                float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
   int err = 0;
   for (int m_base = 0; m_base < M && !err; m_base += 128) {
     const int rows = M - m_base < 128 ? M - m_base : 128;
-    if (rows <= 16) err = launch_nt<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    else if (rows <= 32) err = launch_nt<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    else if (rows <= 64) err = launch_nt<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
-    else err = launch_nt<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, rp, s);
+    if (rows <= 16) err = launch_nt<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    else if (rows <= 32) err = launch_nt<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    else if (rows <= 64) err = launch_nt<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    else err = launch_nt<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
   }
   return err;
 }
 
 template <int AT>
 int launch_epi(const void* A, const bf16_t* W, void* C, int epi, int M, int N, int K, int lda,
-               int ldc, float eps, const RopeEpi& rp, hipStream_t s) {
+               int ldc, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
   switch (epi) {
-    case 0: return launch_rows<AT, 0>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
-    case 1: return launch_rows<AT, 1>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
-    case 2: return launch_rows<AT, 2>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
-    case 3: return launch_rows<AT, 3>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
-    case 4: return launch_rows<AT, 4>(A, W, C, M, N, K, lda, ldc, eps, rp, s);
+    case 0: return launch_rows<AT, 0>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
+    case 1: return launch_rows<AT, 1>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
+    case 2: return launch_rows<AT, 2>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
+    case 3: return launch_rows<AT, 3>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
+    case 4: return launch_rows<AT, 4>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
   }
   return static_cast<int>(hipErrorInvalidValue);
 }
@@ -430,22 +446,24 @@ KVF_EXPORT void kvf_gemm_bf16_set_rows(int rows) { g_rows_override = rows; }
 
 // a_type: 0 = bf16 rows, 1 = fp32 rows normalised by rsqrt(mean(x^2) + eps) in the kernel.
 // epi: 0 store fp32, 1 store bf16, 2 add into fp32, 3 SwiGLU pairs -> bf16 [M, N/2].
-KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, void* C, int epi, int M,
-                             int N, int K, int lda, int ldc, float eps, hipStream_t s) {
+// w_tiled: W is [N, K] row-major (0) or in tiles of 16 x 32 (1, see the head of this file).
+KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, int w_tiled, void* C, int epi,
+                             int M, int N, int K, int lda, int ldc, float eps, hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || epi < 0 || epi > 3 || (epi == 3 && N % 4 != 0))
     return static_cast<int>(hipErrorInvalidValue);
   const RopeEpi none{};
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, none, s);
-  if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, none, s);
+  if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, none, s);
+  if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, none, s);
   return static_cast<int>(hipErrorInvalidValue);
 }
 
 // Fused q/k/v projection with rotary and cache write.  W: [(H + 2*KV) * d, K] with q and k rows
 // permuted so that rotary pairs are neighbouring rows.  q_out: [M, ldq >= H * d] bf16.
-KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, void* q_out, int M,
-                                      int K, int lda, int ldq, float eps, const int* positions,
+KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, int w_tiled,
+                                      void* q_out, int M, int K, int lda, int ldq, float eps,
+                                      const int* positions,
                                       const int* seq_of_token, const float* cos_t,
                                       const float* sin_t, const int* block_table, void* k_pages,
                                       void* v_pages, int H, int KV, int d, int rot, int table_len,
@@ -459,7 +477,7 @@ KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, 
                    table_len, block_size, table_stride, num_blocks, write_kv, n_seqs};
   const int N = (H + 2 * KV) * d;
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, rp, s);
-  if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, rp, s);
+  if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rp, s);
+  if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rp, s);
   return static_cast<int>(hipErrorInvalidValue);
 }

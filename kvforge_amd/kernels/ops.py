@@ -182,7 +182,56 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 # library product there as well.
 SKINNY_MAX_M = 16
 FUSED_NORM_MAX_M = 16
-_GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
+_GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
+
+
+class StreamedWeight:
+    """A bf16 weight matrix ``[N, K]`` kept twice: ``plain`` as the checkpoint has it (what the
+    library product and the fp32 kernels read) and ``tiles``, ``[ceil(N/16), ceil(K/32), 64, 8]``,
+    where tile ``(g, s)`` holds rows ``16g..16g+15``, columns ``32s..32s+31`` in the order the
+    matrix-core instruction takes them (position ``16*c + r`` holds row ``r``, columns
+    ``8c..8c+7``), zero-padded.  The weight-streaming kernel then loads 1 KB of consecutive bytes
+    per operand fragment instead of 64 bytes from each of 16 rows, which is what lets it reach
+    the memory's bandwidth.  Costs the matrix's size in memory a second time."""
+
+    def __init__(self, plain: torch.Tensor) -> None:
+        if plain.dim() != 2 or plain.dtype != BF16 or not plain.is_contiguous():
+            raise KernelError("a streamed weight is a contiguous bf16 matrix")
+        n, k = plain.shape
+        n_pad, k_pad = -(-n // 16) * 16, -(-k // 32) * 32
+        padded = plain
+        if (n_pad, k_pad) != (n, k):
+            padded = torch.zeros(n_pad, k_pad, dtype=BF16, device=plain.device)
+            padded[:n, :k] = plain
+        self.plain = plain
+        self.tiles = (padded.view(n_pad // 16, 16, k_pad // 32, 4, 8).permute(0, 2, 3, 1, 4)
+                      .contiguous().view(n_pad // 16, k_pad // 32, 64, 8))
+        self.shape, self.dtype, self.device = plain.shape, plain.dtype, plain.device
+
+    def dim(self) -> int:
+        return 2
+
+
+TILE_WEIGHTS = True  # parts keep the matrices they stream for few rows in tiles as well
+
+
+def streamed(w: torch.Tensor):
+    """``w`` ready for ``gemm`` and its fused forms: bf16 matrices on the GPU also in tiles."""
+    if (TILE_WEIGHTS and w is not None and w.dtype == BF16 and w.is_cuda and w.dim() == 2
+            and w.is_contiguous()):
+        return StreamedWeight(w)
+    return w
+
+
+def plain_of(w) -> torch.Tensor:
+    return w.plain if isinstance(w, StreamedWeight) else w
+
+
+def _w_args(w) -> tuple[int, int]:
+    """(pointer, tiled flag) of a weight for the weight-streaming kernel."""
+    if isinstance(w, StreamedWeight):
+        return w.tiles.data_ptr(), 1
+    return w.data_ptr(), 0
 
 
 def _gemm_operands(a, w, out, n_out):
@@ -194,7 +243,7 @@ def _gemm_operands(a, w, out, n_out):
         raise KernelError(f"gemm shapes do not agree: a {list(a.shape)}, w {list(w.shape)}, "
                           f"out {list(out.shape)}")
     _check(a, "a", None, None, contiguous=False)
-    _check(w, "w")
+    _check(plain_of(w), "w")
     _check(out, "out", None, None, contiguous=False)
     if a.stride(1) != 1 or out.stride(1) != 1:
         raise KernelError("gemm: rows of a and out must be dense")
@@ -222,10 +271,11 @@ def is_library_product(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0 and m > SKINNY_MAX_M)
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
     """``out = a @ w.T`` (``accumulate``: ``out += a @ w.T`` with ``out`` fp32).
 
-    ``a: [M, K]`` (row stride may exceed K), ``w: [N, K]`` contiguous, ``out: [M, N]``.
+    ``a: [M, K]`` (row stride may exceed K), ``w: [N, K]`` contiguous or a ``StreamedWeight``,
+    ``out: [M, N]``.
     bf16 x bf16 runs on MFMA with fp32 accumulation; any operand in fp32 runs the fp32
     vector-ALU kernel (true 32-bit multiply and accumulate)."""
     m, n, k, lda, ldc = _gemm_operands(a, w, out, lambda n: n)
@@ -239,16 +289,18 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     if a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0:
         if m <= SKINNY_MAX_M:
             f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
-            _ok(f(a.data_ptr(), 0, w.data_ptr(), out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
+            wp, tiled = _w_args(w)
+            _ok(f(a.data_ptr(), 0, wp, tiled, out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
                   _stream()), "gemm_bf16")
         elif accumulate:
             # many rows: the library's bf16 product, then the residual sum in fp32
-            out.add_(torch.mm(a, w.t()))
+            out.add_(torch.mm(a, plain_of(w).t()))
         elif out.dtype == F32:
-            out.copy_(torch.mm(a, w.t()))
+            out.copy_(torch.mm(a, plain_of(w).t()))
         else:
-            torch.mm(a, w.t(), out=out)
+            torch.mm(a, plain_of(w).t(), out=out)
         return
+    w = plain_of(w)
     f = _fn("gemm_generic", "kvf_gemm_generic",
             [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_void_p])
     _ok(f(a.data_ptr(), _tcode(a.dtype), w.data_ptr(), _tcode(w.dtype), out.data_ptr(), out_kind,
@@ -281,7 +333,8 @@ def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: flo
     if m == 0:
         return
     f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
-    _ok(f(a.data_ptr(), 1 if rms else 0, w.data_ptr(), out.data_ptr(), epi, m, n, k, lda, ldc,
+    wp, tiled = _w_args(w)
+    _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, out.data_ptr(), epi, m, n, k, lda, ldc,
           float(rms_eps or 0.0), _stream()), "gemm_bf16")
 
 
@@ -297,7 +350,7 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     rms = rms_eps is not None
     m, k = a.shape
     _check(a, "a", None, (m, k), contiguous=False)
-    _check(w, "w", BF16, ((H + 2 * KV) * d, k))
+    _check(plain_of(w), "w", BF16, ((H + 2 * KV) * d, k))
     if not bf16_kernel_takes(a, w, rms) or a.stride(1) != 1:
         raise KernelError("gemm_qkv_rope: operands do not fit the MFMA kernel")
     _check(q_out, "q_out", BF16, (m, H * d))
@@ -317,9 +370,10 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     if m == 0:
         return
     f = _fn("gemm_bf16", "kvf_gemm_bf16_qkv_rope",
-            [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float]
+            [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float]
             + [c_void_p] * 7 + [c_int] * 10 + [c_void_p])
-    _ok(f(a.data_ptr(), 1 if rms else 0, w.data_ptr(), q_out.data_ptr(), m, k,
+    wp, tiled = _w_args(w)
+    _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, q_out.data_ptr(), m, k,
           a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d, float(rms_eps or 0.0),
           positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(), sin.data_ptr(),
           block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, 2 * half,

@@ -59,6 +59,8 @@ class Transformer:
 
     def load_folder(self, folder: str) -> None:
         load_model_weights(self.spec, folder, self.dtype, self.device)
+        for p in self.spec.all_parts():
+            p.seal()
         self._loaded = True
 
     def kernel_modules(self) -> list[str]:

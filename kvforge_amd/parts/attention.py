@@ -89,7 +89,11 @@ class PagedAttention(Mixer):
         return mods
 
     def num_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in (self.w_qkv, self.w_o) if t is not None)
+        return sum(t.numel() * t.element_size()
+                   for t in map(ops.plain_of, (self.w_qkv, self.w_o)) if t is not None)
+
+    def seal(self) -> None:
+        self.w_qkv, self.w_o = ops.streamed(ops.plain_of(self.w_qkv)), ops.streamed(ops.plain_of(self.w_o))
 
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""

@@ -82,6 +82,10 @@ class Part:
         """Bytes of weights this part reads in one step."""
         return 0
 
+    def seal(self) -> None:
+        """Called once after ``load`` (and any ``absorb_norm``), before the first forward: the
+        place for the last re-layout of weights, such as tiles for the weight-streaming kernel."""
+
     def absorb_norm(self, norm: "Norm") -> bool:
         """Offer the norm that feeds this part.  A part that can apply it inside its own first
         kernel takes what it needs from ``norm`` and returns True; from then on its ``forward``
@@ -158,6 +162,10 @@ class Block(Part):
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
         for p in self.parts():
             p.load(tensors)
+
+    def seal(self) -> None:
+        for p in self.parts():
+            p.seal()
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         out: set[str] = set()

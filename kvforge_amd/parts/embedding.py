@@ -48,7 +48,12 @@ class LMHead(Part):
         return {"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
 
     def num_bytes(self) -> int:
-        return self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
+        w = ops.plain_of(self.weight)
+        return w.numel() * w.element_size() if w is not None else 0
+
+    def seal(self) -> None:
+        # a tied table stays as it is for the embedding; the head streams a tiled copy
+        self.weight = ops.streamed(ops.plain_of(self.weight))
 
     def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
         ops.gemm(x, self.weight, logits)

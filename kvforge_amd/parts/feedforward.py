@@ -50,8 +50,12 @@ class SwiGLU(FeedForward):
         return mods
 
     def num_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in (self.w_gate_up, self.w_down)
-                   if t is not None)
+        return sum(t.numel() * t.element_size()
+                   for t in map(ops.plain_of, (self.w_gate_up, self.w_down)) if t is not None)
+
+    def seal(self) -> None:
+        self.w_gate_up = ops.streamed(ops.plain_of(self.w_gate_up))
+        self.w_down = ops.streamed(ops.plain_of(self.w_down))
 
     def forward(self, x, step, residual) -> None:
         """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""

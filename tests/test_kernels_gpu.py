@@ -161,6 +161,46 @@ def test_gemm_bf16_mfma(m, n, k):
     torch.testing.assert_close(out2.double().cpu(), want, **t32)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n,k", [(352, 96), (40, 2048), (100, 40), (2048, 136), (16, 32)])
+def test_gemm_over_tiled_weights_gives_the_same_bits(m, n, k):
+    """A weight kept in tiles of 16 x 32 (what the parts stream for few rows) gives bit for bit
+    what the row-major matrix gives, in every form of the product: tails in N and K are zero
+    padding inside the tiles; beyond the kernel's rows the row-major copy goes to the library."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    x = (torch.randn(m, k, generator=g) * 2).to(DEV)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16).to(DEV)
+    sw = ops().StreamedWeight(w)
+    assert tuple(sw.tiles.shape) == (-(-n // 16), -(-k // 32), 64, 8) and sw.shape == w.shape
+    # tile (1, 0) or (0, 0), position 16*c + r: row 16g + r, columns 8c..8c+7
+    gi = 1 if n > 16 else 0
+    r, c = min(3, n - 16 * gi - 1), 2 if k >= 24 else 0
+    assert torch.equal(sw.tiles[gi, 0, 16 * c + r], w[16 * gi + r, 8 * c:8 * c + 8])
+    for dt in (torch.float32, torch.bfloat16):
+        o1, o2 = torch.empty(m, n, dtype=dt, device=DEV), torch.empty(m, n, dtype=dt, device=DEV)
+        ops().gemm(a, w, o1)
+        ops().gemm(a, sw, o2)
+        assert torch.equal(o1, o2)
+    res = torch.randn(m, n, generator=g).to(DEV)
+    r1, r2 = res.clone(), res.clone()
+    ops().gemm(a, w, r1, accumulate=True)
+    ops().gemm(a, sw, r2, accumulate=True)
+    assert torch.equal(r1, r2)
+    if n % 4 == 0:
+        g1 = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
+        g2 = torch.empty_like(g1)
+        ops().gemm_fused(x, w, g1, rms_eps=1e-5, silu_pairs=True)
+        ops().gemm_fused(x, sw, g2, rms_eps=1e-5, silu_pairs=True)
+        assert torch.equal(g1, g2)
+    # many rows: the library reads the row-major copy
+    big = torch.randn(40, k, generator=g).to(torch.bfloat16).to(DEV)
+    o1, o2 = torch.empty(40, n, device=DEV), torch.empty(40, n, device=DEV)
+    ops().gemm(big, w, o1)
+    ops().gemm(big, sw, o2)
+    assert torch.equal(o1, o2)
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 20])
 @pytest.mark.parametrize("n,k", [(352, 96), (512, 2048), (48, 40)])
 def test_gemm_fused_norm_and_gate(m, n, k):
@@ -239,6 +279,11 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     q = torch.empty(m, H * d, dtype=torch.bfloat16, device=DEV)
     ops().gemm_qkv_rope(a, w, q, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV), kp,
                         vp, H, KV, d, rms_eps=eps if rms else None)
+    # the same over the weight in tiles: the same bits
+    kp_t, vp_t, q_t = torch.zeros_like(kp_ref), torch.zeros_like(vp_ref), torch.empty_like(q)
+    ops().gemm_qkv_rope(a, ops().StreamedWeight(w), q_t, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t,
+                        table.to(DEV), kp_t, vp_t, H, KV, d, rms_eps=eps if rms else None)
+    assert torch.equal(q_t, q)
     # the fused kernel rotates fp32 accumulators, the reference rounds the projection to bf16
     # first; with fp32 rows the rounding of the normalised input differs as well
     t = dict(atol=3e-2, rtol=3e-2)

@@ -77,6 +77,7 @@ def test_swiglu_part(dtype):
          "m.down_proj.weight": rand(48, 112, seed=5, scale=0.2).to(dtype)}
     assert {k: v.shape for k, v in part.weight_specs().items()} == {k: tuple(v.shape) for k, v in w.items()}
     part.load({k: v.to(DEV) for k, v in w.items()})
+    part.seal()
     x = rand(9, 48, seed=6).to(dtype)
     res = rand(9, 48, seed=7)
     step = Step()
@@ -123,6 +124,7 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
          "a.v_proj.weight": rand(KV * d, hidden, seed=12, scale=0.15).to(dtype),
          "a.o_proj.weight": rand(hidden, H * d, seed=13, scale=0.1).to(dtype)}
     part.load({k: v.to(DEV) for k, v in w.items()})
+    part.seal()
     cache = CacheManager(bs, [CacheGroup((0,), KV, d, window)], 24)
     ls = LayerState(group=0, owns_cache=True,
                     k_pages=torch.zeros(24, KV, bs, d, dtype=dtype, device=DEV),
@@ -171,6 +173,7 @@ def test_pre_norm_block(dtype, n):
         t = torch.randn(spec.shape, generator=g) * (0.1 if spec.init == "norm" else 0.15)
         w[name] = (t + 1 if spec.init == "norm" else t).to(dtype)
     block.load({k: v.to(DEV) for k, v in w.items()})
+    block.seal()
     x = rand(n, hidden, seed=21)
     cache = CacheManager(4, [CacheGroup((0,), KV, d, None)], 8)
     cache.allocate("r", n)
