@@ -445,7 +445,9 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
   if (seq < 0 || seq >= a.n_seqs) return;
   const int kvh = blockIdx.y / chunks, tile = blockIdx.y - kvh * chunks;
-  const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
+  // without cu_q every sequence has one token, its own: nothing then waits for a load before the
+  // query and the page lookups can be asked for
+  const int q0 = cu_q ? cu_q[seq] : seq, qlen = cu_q ? cu_q[seq + 1] - q0 : 1, ctx = ctx_lens[seq];
   const int start = ctx - qlen;
   const bool seq_ok = qlen > 0 && start >= 0;
   const Pages pg{k_pages, vt_pages, block_table + static_cast<size_t>(seq) * a.table_stride, kvh, ctx,
@@ -594,7 +596,7 @@ __global__ __launch_bounds__(64) void attn_split_combine_kernel(
     m = ml.x;
     l = ml.y;
   }
-  const int tok = cu_q[seq];
+  const int tok = cu_q ? cu_q[seq] : seq;
   const float mm = wave_max(m);
   const float c = m == -INFINITY ? 0.f : exp2f(m - mm);
   const float ll = wave_sum(l * c);
@@ -694,7 +696,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
 }
 
 // Single-token queries: sequences seq_ids[0..num_seqs) (or 0..num_seqs-1), key range cut into
-// `splits`.  With splits > 1, part_acc holds num_seqs*H*splits*d floats and part_ml
+// `splits`.  cu_q may be null when the token of sequence i is token i.  With splits > 1, part_acc holds num_seqs*H*splits*d floats and part_ml
 // num_seqs*H*splits*2; calls that share them must not overlap.
 KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const void* vt_pages,
                                     const int* block_table, const int* seq_ids, const int* cu_q,

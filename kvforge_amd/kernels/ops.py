@@ -469,13 +469,18 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 block_table: torch.Tensor, seq_ids: torch.Tensor | None, num_seqs: int,
                 cu_q: torch.Tensor, ctx_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
-                workspace: tuple[torch.Tensor, torch.Tensor] | None = None) -> None:
+                workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
+                token_is_seq: bool = False) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  On the
     matrix cores the key range may be cut into ``splits`` runs; ``workspace`` then holds fp32
-    partial accumulators and fp32 (max, sum) pairs.  The vector-ALU kernel ignores ``splits``."""
+    partial accumulators and fp32 (max, sum) pairs.  The vector-ALU kernel ignores ``splits``.
+    ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
+    single tokens), which spares the matrix-core kernel a dependent load."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    if token_is_seq and seq_ids is not None:
+        raise KernelError("attn_decode: token_is_seq is for batches where every sequence decodes")
     if seq_ids is not None:
         _check(seq_ids, "seq_ids", I32, (None,))
         if seq_ids.shape[0] < num_seqs:
@@ -499,7 +504,8 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
             [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
-          seq_ids.data_ptr() if seq_ids is not None else None, cu_q.data_ptr(),
+          seq_ids.data_ptr() if seq_ids is not None else None,
+          None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
           block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs, int(splits),

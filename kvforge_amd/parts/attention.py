@@ -134,5 +134,6 @@ class PagedAttention(Mixer):
             splits, workspace = step.decode_plan(H, KV, d, window)
             ops.attn_decode(qkv, layer.k_pages, layer.v_pages, table, step.decode_seq_ids,
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
-                            window, splits, workspace)
+                            window, splits, workspace,
+                            token_is_seq=step.decode_seq_ids is None and work is None)
         add_product(step, out, self.w_o, residual)

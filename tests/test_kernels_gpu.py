@@ -437,6 +437,12 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, n,
                       cu.to(DEV), ctx.to(DEV), out, H, KV, d, scale, window, splits, ws)
     torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    # the caller may vouch that token i is sequence i's: the same bits without the lookup
+    same = torch.zeros_like(out)
+    ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, n,
+                      cu.to(DEV), ctx.to(DEV), same, H, KV, d, scale, window, splits, ws,
+                      token_is_seq=True)
+    assert torch.equal(same, out)
     # a subset of the sequences, named by seq_ids; the others stay untouched
     ids = torch.tensor([4, 1], dtype=torch.int32)
     out2 = torch.full((n, H * d), 5.0, dtype=dtype, device=DEV)
