@@ -176,11 +176,12 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 
 
 # ------------------------------------------------------------------------------ matrix products
-# Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16: one
-# 16-row tile.  With more rows the library's bf16 product measured faster on every shape of a
-# 1B-parameter decoder (it splits K across workgroups), and the reference's engine uses a
-# library product there as well.
-SKINNY_MAX_M = 16
+# Rows of the left operand up to which the weight-streaming MFMA kernel is used for bf16.  Over
+# tiled weights it measured faster than the library's product up to 32 rows on the shapes of a
+# 1B-parameter decoder (and it folds rotary, cache write, SwiGLU gate and residual sum into its
+# store); with more rows the library wins, and the reference's engine uses a library product
+# there as well.
+SKINNY_MAX_M = 32
 FUSED_NORM_MAX_M = 16
 _GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
 

@@ -365,23 +365,24 @@ def test_graph_replay_equals_eager_steps(model_b, dtype):
     assert graphed == eager
 
 
-def test_graph_replay_with_many_requests(model_a):
-    """Twenty-four requests decode together: the padded batch is 32, past the 16 rows the
-    hand-written matrix product takes, so the captured graph holds the library's products; its
-    replays must give the tokens of eager launches."""
+@pytest.mark.parametrize("count,bucket", [(24, 32), (40, 64)])
+def test_graph_replay_with_many_requests(model_a, count, bucket):
+    """Many requests decode together.  A padded batch of 32 is two row tiles of the hand-written
+    matrix product; one of 64 is past what it takes, so the captured graph holds the library's
+    products.  Replays must give the tokens of eager launches either way."""
     folder, oracle = model_a
-    prompts = prompts_for(256, 24, 12, 4, 20)
+    prompts = prompts_for(256, count, 12, 4, 20)
     params = SamplingParams(max_tokens=14, temperature=0.0)
 
     def run(use_graphs):
-        engine = engine_for(folder, "bfloat16", block_size=8, max_num_seqs=32,
-                            max_num_batched_tokens=128, use_graphs=use_graphs)
+        engine = engine_for(folder, "bfloat16", block_size=8, max_num_seqs=64, num_blocks=512,
+                            max_num_batched_tokens=256, use_graphs=use_graphs)
         outs = engine.generate(prompts, params)
         return [o.output_token_ids for o in outs], engine
 
     eager, _ = run(False)
     graphed, engine = run(True)
-    assert any(b == 32 for b, _ in engine.runner.graphs) and engine.runner.num_graph_replays >= 8
+    assert any(b == bucket for b, _ in engine.runner.graphs) and engine.runner.num_graph_replays >= 8
     assert graphed == eager
     for p, out in zip(prompts, graphed):
         oracle.check_choices(p, out, 3e-2)
