@@ -17,7 +17,7 @@ constexpr int ROWS = 16;
 
 struct AttnArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs;
-  int tiles_per_seq;  // 0: `work` holds (sequence, tile) pairs; > 0: `work` lists sequences (or
+  int tiles_per_seq;  // 0: `work` holds (sequence, tile, tile or -1) rows; > 0: `work` lists sequences (or
                       // is null for 0, 1, 2, ...) and each takes this many tiles
   float scale;
 };
@@ -38,8 +38,11 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
     seq = work ? work[idx] : idx;
     tile = blockIdx.x - idx * a.tiles_per_seq;
   } else {
-    seq = work[2 * blockIdx.x];
-    tile = work[2 * blockIdx.x + 1];
+    // rows (sequence, tile, tile or -1): two workgroups per row, one for each tile
+    const int w = blockIdx.x >> 1;
+    seq = work[3 * w];
+    tile = work[3 * w + 1 + (blockIdx.x & 1)];
+    if (tile < 0) return;
   }
   if (seq < 0 || seq >= a.n_seqs) return;
   const int kvh = blockIdx.y;
@@ -196,7 +199,7 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
 }  // namespace
 
 // dtype: 0 = fp32, 1 = bf16.  d must be a multiple of 16 and at most 256 (checked by the caller
-// and here).  tiles_per_seq == 0: `work` holds num_work pairs (sequence, 16-row tile).
+// and here).  tiles_per_seq == 0: `work` holds num_work rows (sequence, 16-row tile, tile or -1).
 // tiles_per_seq > 0: num_work sequences, listed in `work` or 0..num_work-1 when it is null, each
 // with that many tiles (single-token queries need ceil(G / 16)).
 KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, const void* v_pages,
@@ -210,7 +213,7 @@ KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, c
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
              tiles_per_seq, scale};
-  if (tiles_per_seq > 0) num_work *= tiles_per_seq;
+  num_work *= tiles_per_seq > 0 ? tiles_per_seq : 2;
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)

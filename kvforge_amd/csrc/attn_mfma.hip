@@ -281,17 +281,20 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KVF_WAVE);  // the same in all lanes
   const int j16 = lane % 16, kg = lane / 16;
   const int G = a.H / a.KV, D = a.d;
-  // The kv heads of the upper half of the grid walk the work list backwards: where two
-  // workgroups half a grid apart land on one compute unit, a long run of keys meets a short one.
-  const int wi = blockIdx.y >= (gridDim.y + 1) / 2 ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
-  const int seq = work[2 * wi], kvh = blockIdx.y;
+  // A work row names a sequence and up to two of its items (the second may be -1), which the
+  // workgroup takes one after the other: the host pairs an early item (few keys to walk) with a
+  // late one (many), so that under the causal mask all workgroups have about the same to do.
+  const int seq = work[3 * blockIdx.x], kvh = blockIdx.y;
   if (seq < 0 || seq >= a.n_seqs) return;
   const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
   const int start = ctx - qlen;
   const bool seq_ok = qlen > 0 && start >= 0;
-  const int wg_tile = work[2 * wi + 1] * WAVES * RT;
   const Pages pg{k_pages, vt_pages, block_table + static_cast<size_t>(seq) * a.table_stride, kvh, ctx,
                  j16, kg};
+  for (int part = 0; part < 2; ++part) {
+  const int item = work[3 * blockIdx.x + 1 + part];
+  if (item < 0) continue;
+  const int wg_tile = item * WAVES * RT;
 
   Rows<RT> rows;
   bf16x8 qf[RT][DC];
@@ -328,22 +331,45 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     // fragment f of a block: K (tile f / DC, step f % DC) for f < N_K, then V^T element tiles;
     // wave w stages fragments w, w + 4, ...
     const int kb_first = (lo_g / 32) * 32;
+    // What does not change from block to block is worked out once per fragment: the key a lane
+    // reads relative to the block's start, and its offset inside a page apart from the key's slot
+    // (in fragments of 16 bytes).
     uint4 stage[FPW];
     PageRef page[FPW];
     int live[FPW];
+    int key_off[FPW];
+    unsigned lane_off[FPW];
+    bool is_k[FPW], whole[FPW];
+    const unsigned page_stride = static_cast<unsigned>(a.KV) * a.bs * (D / 8);
+#pragma unroll
+    for (int i = 0; i < FPW; ++i) {
+      const int f = wave + i * WAVES;
+      is_k[i] = f < N_K;
+      if (is_k[i]) {
+        const int t = f / DC, c = f % DC;
+        key_off[i] = 8 * (j16 >> 2) + 4 * t + (j16 & 3);
+        whole[i] = !((DT % 2) && c == DT / 2 && kg >= 2);  // a step that reaches past d
+        lane_off[i] = static_cast<unsigned>(kvh) * a.bs * (D / 8) + (whole[i] ? c * 4 + kg : 0);
+      } else {
+        key_off[i] = 8 * kg;
+        whole[i] = f < N_FRAG;
+        lane_off[i] = (static_cast<unsigned>(kvh) * D + (f - N_K) * 16 + j16) * (a.bs / 8);
+      }
+    }
     auto locate = [&](int kb) {
 #pragma unroll
-      for (int i = 0; i < FPW; ++i) {
-        const int f = wave + i * WAVES;
-        page[i] = f < N_K ? k_page(pg, a, kb, f / DC) : v_page(pg, a, kb);
-      }
+      for (int i = 0; i < FPW; ++i) page[i] = page_of_key(pg, a, kb + key_off[i]);
     };
     auto fetch = [&](int kb) {
 #pragma unroll
       for (int i = 0; i < FPW; ++i) {
-        const int f = wave + i * WAVES;
-        if (f < N_K) stage[i] = k_fragment<DT>(pg, a, kb, f / DC, f % DC, page[i], live[i]);
-        else if (f < N_FRAG) stage[i] = v_fragment(pg, a, kb, f - N_K, page[i], live[i]);
+        const int key = kb + key_off[i];
+        const unsigned slot = static_cast<unsigned>(key - block_of(a, key) * a.bs);
+        const bool ok = page[i].ok(a.nb) && whole[i];
+        live[i] = !ok ? 0 : is_k[i] ? 8 : min(ctx - key, 8);
+        const unsigned off = __umul24(ok ? page[i].page : 0, page_stride) + lane_off[i] +
+                             (is_k[i] ? __umul24(slot, D / 8) : slot >> 3);
+        stage[i] = ld16((is_k[i] ? k_pages : vt_pages) + static_cast<size_t>(off) * 8);
       }
     };
     auto put = [&](int buf) {
@@ -423,6 +449,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 #pragma unroll
     for (int t = 0; t < DT; ++t) *reinterpret_cast<uint2*>(o + t * 16) = pack4(acc[rt][t], inv);
   }
+  __syncthreads();  // the staging buffers are free for the next item
+  }  // part
 }
 
 // ------------------------------------------------------------------------- few rows, split keys
@@ -617,13 +645,15 @@ bool args_ok(int H, int KV, int d, int bs, int nb, int table_stride, float scale
   if (!(d > 0 && d % 16 == 0 && d <= 256 && KV > 0 && H % KV == 0 && bs > 0 && bs % 8 == 0)) return false;
   if (nb < 1 || table_stride < 1 || !(scale > 0.f)) return false;
   const unsigned long long limit = 1ull << 32;
+  // (the page number and a page's size in fragments also go through 24-bit multiplies)
   return static_cast<unsigned long long>(table_stride) * bs * bs < limit &&
-         static_cast<unsigned long long>(nb) * KV * bs * d / 8 < limit;
+         static_cast<unsigned long long>(nb) * KV * bs * d / 8 < limit && nb < (1 << 24) &&
+         static_cast<unsigned long long>(KV) * bs * d / 8 < (1ull << 24);
 }
 unsigned magic_of(int bs) { return static_cast<unsigned>((1ull << 32) / bs) + 1u; }
 
 // Row tiles per wave and LDS sharing by head size: what fits the registers and 64 KB of LDS.
-constexpr int runs_rt(int dt) { return dt <= 8 ? 2 : 1; }
+constexpr int runs_rt(int) { return 1; }  // paired items balance the work; one tile per wave keeps more workgroups in flight
 constexpr bool runs_share(int dt) { return dt <= 12; }
 
 template <int DT>
@@ -674,7 +704,7 @@ void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, 
 // Rows of a query run one workgroup takes: 4 waves x RT tiles x 16 rows.
 KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d) { return WAVES * runs_rt(d / 16) * 16; }
 
-// Query runs: `work` holds num_work pairs (sequence, item) where item i covers rows
+// Query runs: `work` holds num_work rows (sequence, item, item or -1) where item i covers rows
 // [i * rows_per_item, (i + 1) * rows_per_item) of the sequence's qlen * H/KV rows per kv head.
 KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const void* vt_pages,
                                      const int* block_table, const int* cu_q, const int* ctx_lens,

@@ -183,17 +183,21 @@ class Step:
 
     def prefill_work(self, group_size: int, rows_per_item: int = ROWS_PER_TILE
                      ) -> torch.Tensor | None:
-        """``[num_work, 2]`` (sequence row, item) for every query run longer than one token: a
-        run of ``q`` tokens has ``q * group_size`` rows per kv head, an item covers
-        ``rows_per_item`` of them."""
+        """``[num_work, 3]`` rows (sequence row, item, item or -1) for every query run longer than
+        one token: a run of ``q`` tokens has ``q * group_size`` rows per kv head, an item covers
+        ``rows_per_item`` of them, and a workgroup takes the items of one row one after the other.
+        Item ``i`` is paired with item ``n - 1 - i``: under the causal mask the early one walks
+        few keys and the late one many, so every pair has about the same to do."""
         if not self.prefill_seqs:
             return None
         key = (group_size, rows_per_item)
         w = self._work.get(key)
         if w is None:
-            pairs = [(b, t) for b in self.prefill_seqs
-                     for t in range(-(-self.q_lens[b] * group_size // rows_per_item))]
-            w = torch.tensor(pairs, dtype=torch.int32).reshape(-1, 2).to(self.device)
+            rows = []
+            for b in self.prefill_seqs:
+                n = -(-self.q_lens[b] * group_size // rows_per_item)
+                rows += [(b, i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
+            w = torch.tensor(rows, dtype=torch.int32).reshape(-1, 3).to(self.device)
             self._work[key] = w
         return w
 

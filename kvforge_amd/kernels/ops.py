@@ -425,7 +425,7 @@ def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
 def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int) -> int:
     """Rows of (query token, head in group) that one entry of a prefill work list covers."""
     if attention_on_matrix_cores(dtype, block_size):
-        return 128 if head_dim <= 128 else 64
+        return int(_fn("attn_mfma", "kvf_attn_mfma_rows_per_item", [c_int])(int(head_dim)))
     return 16
 
 
@@ -433,13 +433,14 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, window: int = 0) -> None:
-    """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 2]`` pairs
-    (sequence row, item) where a sequence has ``query_len * H/KV`` rows per kv head and an item
-    covers ``prefill_rows_per_item(...)`` of them.  ``v_pages`` are transposed:
+    """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
+    (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
+    an item covers ``prefill_rows_per_item(...)`` of them, and the items of one row are taken by
+    one workgroup in turn (pair an early item with a late one).  ``v_pages`` are transposed:
     ``[num_blocks, KV, head_dim, block_size]``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
-    _check(work, "work", I32, (None, 2))
+    _check(work, "work", I32, (None, 3))
     nb, _, bs, _ = k_pages.shape
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",

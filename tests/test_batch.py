@@ -40,7 +40,9 @@ def test_flat_varlen_batch_reference_vector():
         slot = int(step.block_tables[0][s, p // 4]) * 4 + p % 4
         assert slot == cache.slot("ab"[s], p)
     assert step.n_decode == 1 and step.decode_seq_ids.tolist() == [1] and step.prefill_seqs == [0]
-    assert step.prefill_work(2).tolist() == [[0, 0]] and step.prefill_work(6).tolist() == [[0, 0], [0, 1]]
+    # 3 tokens x group size over 16-row items: one item, then two paired into one row
+    assert step.prefill_work(2).tolist() == [[0, 0, -1]] and step.prefill_work(6).tolist() == [[0, 0, 1]]
+    assert step.prefill_work(6, 4).tolist() == [[0, 0, 4], [0, 1, 3], [0, 2, -1]]
 
 
 def test_wanted_places_and_modes():

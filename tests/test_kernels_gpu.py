@@ -372,12 +372,15 @@ def attn_reference(paged, q, seq_lens, q_lens, scale, window):
 
 
 def prefill_work(q_lens, G, dtype=torch.float32, d=16, bs=4):
+    """Rows (sequence, item, item or -1): an early item paired with a late one, as the engine
+    does; the odd one out of three is left alone."""
     rows = ops().prefill_rows_per_item(dtype, d, bs)
     work = []
     for s, ql in enumerate(q_lens):
-        for t in range(-(-ql * G // rows)):
-            work.append((s, t))
-    return torch.tensor(work, dtype=torch.int32).reshape(-1, 2)
+        n = -(-ql * G // rows)
+        for t in range((n + 1) // 2):
+            work.append((s, t, n - 1 - t if n - 1 - t > t else -1))
+    return torch.tensor(work, dtype=torch.int32).reshape(-1, 3)
 
 
 # the (context, query) cases of the reference's tests/test_paged_attention.py:60-66 and more
