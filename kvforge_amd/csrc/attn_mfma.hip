@@ -27,11 +27,14 @@
 // Loads are never predicated: a lane without a valid page reads page 0 and its fragment is
 // cleared by a mask when it is consumed, so nothing waits on a load before its data is needed.
 //
-// Query runs: a workgroup takes 4 * RT consecutive row tiles of one (sequence, kv head) from a
-//   work list.  Three stages are in flight: page lookups two blocks ahead, fragment loads one
-//   block ahead (registers, then the other half of a double LDS buffer), products of this block.
+// Query runs: an item is 4 * RT consecutive row tiles of one (sequence, kv head), one tile set per
+//   wave; a workgroup takes the items of a work row in turn: the host pairs an early item with a
+//   late one, so that under the causal mask every workgroup walks about as many keys.  Three
+//   stages are in flight: page lookups two blocks ahead, fragment loads one block ahead
+//   (registers, then the other half of a double LDS buffer), products of this block.
 // Few rows, long key range: a workgroup takes one row tile and one of `splits` cuts of the key
-//   range; its four waves take the blocks of that cut in turn and are merged through LDS; with
+//   range; its waves (eight, or four where the grid fills the chip) take the blocks of that cut in
+//   turn and are merged through LDS; with
 //   splits > 1 partial (max, sum, accumulator) go to a workspace that
 //   `attn_split_combine_kernel` merges in split order.
 // block_size must be a multiple of 8 (a lane's eight keys lie in one page), d a multiple of 16;
