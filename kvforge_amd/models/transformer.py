@@ -87,12 +87,12 @@ class Transformer:
 
     @property
     def weight_bytes(self) -> int:
-        seen: dict[int, int] = {}
-        for p in self.spec.all_parts():
-            for t in vars(p).values():
-                if isinstance(t, torch.Tensor) and t.is_floating_point() and t.dim() >= 1:
-                    seen[t.data_ptr()] = t.numel() * t.element_size()
-        return sum(seen.values())
+        """Bytes of weights one decode step reads: what every part says it reads (``num_bytes``),
+        a block once for each time the run order names it.  An embedding table counts only where
+        a head reads it whole."""
+        spec = self.spec
+        total = sum(p.num_bytes() for p in (spec.embedding, spec.final_norm, spec.head, *spec.positions))
+        return total + sum(spec.blocks[c.layer].num_bytes() for c in self.order)
 
     # ------------------------------------------------------------------ forward
     def forward(self, step) -> torch.Tensor:
