@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512]
                     [--dtype bfloat16] [--layers L] [--no-points] [--phase all|decode|prefill]
+                    [--preset llama-1b|llama-3b|llama-8b] [--context-len 8192]
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -31,9 +32,11 @@ MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 CONTEXT_CAP = 8192
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
+MODEL_NAMES = {"llama-1b": "Llama 3.2 1B", "llama-3b": "Llama 3.2 3B", "llama-8b": "Llama 3.1 8B"}
 
 
-def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True, run_steps=None):
+def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True, run_steps=None,
+                 context_cap=CONTEXT_CAP):
     import kvforge_amd
     from kvforge_amd import CacheConfig, EngineConfig, InferenceEngine, SchedulerConfig
 
@@ -41,7 +44,7 @@ def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True
     cfg = EngineConfig(
         cache=CacheConfig(block_size=BLOCK_SIZE, num_blocks=num_blocks, watermark=0.0),
         scheduler=SchedulerConfig(max_num_seqs=max_num_seqs, max_num_batched_tokens=PREFILL_TOKENS,
-                                  max_model_len=CONTEXT_CAP),
+                                  max_model_len=context_cap),
         dtype=dtype, use_graphs=use_graphs)
     if run_steps is not None:
         cfg.decode_run_steps = run_steps
@@ -54,12 +57,20 @@ def random_prompts(vocab, n, length, seed):
     return [torch.randint(1, vocab, (length,), generator=g).tolist() for _ in range(n)]
 
 
+def early_tokens(batch, prompt_len):
+    """Most tokens a request decodes before the last prompt of the batch has been read."""
+    return -(-batch * prompt_len // PREFILL_TOKENS) + 1
+
+
 def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
     """Prefill ``batch`` prompts, run ``warmup`` decode steps untimed, then time ``steps``."""
     import torch
     from kvforge_amd import SamplingParams
 
-    params = SamplingParams(max_tokens=steps + warmup + 8, temperature=0.0, ignore_eos=True)
+    # requests admitted first decode while the later prompts are still being read: leave them
+    # room for that, so that every request lives through the timed steps
+    params = SamplingParams(max_tokens=steps + warmup + early_tokens(batch, prompt_len) + 8,
+                            temperature=0.0, ignore_eos=True)
     for p in random_prompts(vocab, batch, prompt_len, seed):
         engine.add_request(p, params)
     while any(r.is_prefill for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
@@ -78,6 +89,7 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
         return produced
 
     decode_steps(warmup)
+    assert len(engine.scheduler.running) == batch
     ctx_start = [r.num_tokens for r in engine.scheduler.running]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -85,6 +97,7 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ctx_end = [r.num_tokens for r in engine.scheduler.running]
+    assert len(ctx_end) == batch and produced == batch * steps, (len(ctx_end), produced)
     for rid in list(engine.scheduler.requests):
         engine.abort_request(rid)
     mean_ctx = (sum(ctx_start) + sum(ctx_end)) / 2.0 / max(1, batch)
@@ -126,6 +139,10 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=512)
     ap.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
+    ap.add_argument("--preset", choices=["llama-1b", "llama-3b", "llama-8b"], default="llama-1b",
+                    help="layer sizes of the model (random weights); the default is the headline run")
+    ap.add_argument("--context-len", type=int, default=CONTEXT_CAP,
+                    help="longest request the engine admits (prompt and new tokens)")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graphs", action="store_true")
@@ -141,7 +158,7 @@ def main() -> int:
     import torch
     import kvforge_amd
 
-    cfg = kvforge_amd.preset_dict("llama-1b")
+    cfg = kvforge_amd.preset_dict(args.preset)
     full_layers = cfg["num_hidden_layers"]
     layers_run = args.layers or full_layers
     cfg["num_hidden_layers"] = layers_run
@@ -156,9 +173,10 @@ def main() -> int:
         batches = [args.batch] + ([b for b in (1, 64) if b != args.batch] if points else [])
         prefill_s = None
         for b in batches:
-            need = b * (args.prompt_len + args.steps + args.warmup + 16)
+            need = b * (args.prompt_len + args.steps + args.warmup + early_tokens(b, args.prompt_len) + 16)
             engine = build_engine(folder, args.dtype, max(b, 1), max(need, PREFILL_TOKENS + 64),
-                                  use_graphs=not args.no_graphs, run_steps=args.decode_run_steps)
+                                  use_graphs=not args.no_graphs, run_steps=args.decode_run_steps,
+                                  context_cap=args.context_len)
             if args.phase != "prefill":
                 results[b] = decode_run(engine, vocab, b, args.prompt_len, args.steps, args.warmup)
             if b == args.batch:
@@ -182,20 +200,21 @@ def main() -> int:
     prefill_flops = (2.0 * n * nums["linear_params"] + 2.0 * nums["head_params"]
                      + 2.0 * n * n * nums["attn_hd"] * layers_run)
     line = {
-        "metric": "decode tok/s (Llama 3.2 1B shape, batch %d)" % args.batch,
+        "metric": "decode tok/s (%s shape, batch %d)" % (MODEL_NAMES[args.preset], args.batch),
         "value": round(main_run["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(main_run["ms_per_step"], 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random weights N(0, 0.02), uniform-random token ids",
         "config": {
-            "model": "llama-3.2-1b-shape", "layers": full_layers, "layers_run": layers_run,
+            "model": MODEL_NAMES[args.preset].lower().replace(" ", "-") + "-shape", "layers": full_layers, "layers_run": layers_run,
             "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
-            "intermediate": cfg["intermediate_size"], "vocab": vocab, "tied_embeddings": True,
-            "rope": "theta 5e5, llama3 factor 32", "rms_norm_eps": cfg["rms_norm_eps"],
+            "intermediate": cfg["intermediate_size"], "vocab": vocab,
+            "tied_embeddings": cfg["tie_word_embeddings"],
+            "rope": "theta %.0e, llama3 factor %g" % (cfg["rope_theta"], cfg["rope_scaling"]["factor"]), "rms_norm_eps": cfg["rms_norm_eps"],
             "global_batch": args.batch, "seq_len": args.prompt_len, "new_tokens": args.steps + 1,
-            "context_len": CONTEXT_CAP, "block_size": BLOCK_SIZE, "parallelism": "single-gpu",
+            "context_len": args.context_len, "block_size": BLOCK_SIZE, "parallelism": "single-gpu",
             "sampling": "greedy", "decode_run_steps": run_steps_used,
         },
         "prefill": {"value": round(n / prefill_s, 1), "tokens": n, "ms": round(prefill_s * 1e3, 3),
