@@ -53,8 +53,9 @@ class ModelRunner:
         self._windowed = [g.window is not None for g in groups]
         self.num_forward_passes = 0
         self.num_tokens_processed = 0
-        # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph
-        self.use_graphs = bool(use_graphs)
+        # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph;
+        # only if every part's launches may be replayed for another batch
+        self.use_graphs = bool(use_graphs) and all(p.replayable for p in model.spec.all_parts())
         self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
         self.num_graph_replays = 0
         cap = self.meta.max_seqs

@@ -22,6 +22,7 @@ from kvforge_amd.registry import register_mixer
 class PagedAttention(Mixer):
     """``window``: ``None`` attends to every earlier position, ``w`` to the last ``w``."""
 
+    replayable = True
     settles_residual = True  # its norm kernel adds what is owed to the stream
 
     def __init__(self, prefix: str, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,

@@ -69,6 +69,12 @@ class Part:
 
     prefix: str = ""
 
+    # Whether ``forward`` only launches device work whose arguments live in the step's device
+    # buffers, so that a launch captured for one batch may be replayed for another.  A part that
+    # looks at the step's host-side fields (lengths, slot numbers) or waits for the device is
+    # not; one such part keeps the whole model out of the captured decode path.
+    replayable: bool = False
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {}
 
@@ -175,6 +181,10 @@ class Block(Part):
 
     def num_bytes(self) -> int:
         return sum(p.num_bytes() for p in self.parts())
+
+    @property
+    def replayable(self) -> bool:
+        return all(p.replayable for p in self.parts())
 
 
 def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor) -> None:

@@ -11,6 +11,8 @@ from kvforge_amd.parts.base import Part, WeightSpec
 class TokenEmbedding(Part):
     """``h0 = table[ids]`` into the fp32 residual stream; no scaling."""
 
+    replayable = True
+
     def __init__(self, prefix: str, vocab: int, hidden: int) -> None:
         self.prefix, self.vocab, self.hidden = prefix, int(vocab), int(hidden)
         self.table: torch.Tensor | None = None
@@ -31,6 +33,8 @@ class TokenEmbedding(Part):
 class LMHead(Part):
     """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
     table when the head shares it (then no tensor of its own is expected)."""
+
+    replayable = True
 
     def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None) -> None:
         self.prefix, self.vocab, self.hidden, self.tied_to = prefix, int(vocab), int(hidden), tied_to

@@ -11,6 +11,7 @@ from kvforge_amd.registry import register_feed_forward
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    replayable = True
     settles_residual = True  # its norm kernel adds what is owed to the stream
 
     def __init__(self, prefix: str, hidden: int, intermediate: int) -> None:

@@ -13,6 +13,8 @@ from kvforge_amd.registry import register_norm
 class RMSNorm(Norm):
     """``y = x * rsqrt(mean(x^2) + eps) * weight`` in fp32, rounded once to the output type."""
 
+    replayable = True
+
     def __init__(self, prefix: str, width: int, eps: float) -> None:
         self.prefix, self.width, self.eps = prefix, int(width), float(eps)
         self.weight: torch.Tensor | None = None

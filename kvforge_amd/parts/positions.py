@@ -42,6 +42,8 @@ class RotaryPositions(Positions):
     """Half-split rotary pairs (element ``i`` with ``i + rot_dim/2``) over the first ``rot_dim``
     elements of each head."""
 
+    replayable = True
+
     def __init__(self, rot_dim: int, theta: float, scaling: RopeScaling | None = None) -> None:
         if rot_dim <= 0 or rot_dim % 2:
             raise ValueError(f"rotary width must be positive and even, got {rot_dim}")
