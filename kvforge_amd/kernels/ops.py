@@ -183,6 +183,7 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 # there as well.
 SKINNY_MAX_M = 32
 FUSED_NORM_MAX_M = 16
+FUSED_EPILOGUE_MAX_M = 64
 _GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
 
 
@@ -253,23 +254,31 @@ def _gemm_operands(a, w, out, n_out):
     return m, n, k, lda, ldc
 
 
-def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False) -> bool:
+def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False,
+                      fused_epilogue: bool = False) -> bool:
     """Whether the MFMA weight-streaming kernel takes these operands: bf16 weights, bf16 rows
     (or, with ``rms``, fp32 rows), 16-byte aligned rows, at most ``SKINNY_MAX_M`` of them.
     Folding the norm in pays only while every workgroup converts one tile of rows
-    (``FUSED_NORM_MAX_M``); beyond that a norm kernel of its own is cheaper."""
+    (``FUSED_NORM_MAX_M``); beyond that a norm kernel of its own is cheaper.  Where the kernel's
+    epilogue stands for a kernel of its own after the library's product (``fused_epilogue``:
+    rotary and cache write, the SwiGLU gate) it pays up to ``FUSED_EPILOGUE_MAX_M`` rows."""
     m, k = a.shape
     lda = a.stride(0) if m > 1 else k
+    limit = FUSED_NORM_MAX_M if rms else (FUSED_EPILOGUE_MAX_M if fused_epilogue else SKINNY_MAX_M)
     return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and k % 8 == 0 and lda % 8 == 0
-            and m <= (FUSED_NORM_MAX_M if rms else SKINNY_MAX_M))
+            and m <= limit)
 
 
 def is_library_product(a: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether ``gemm(a, w, ...)`` hands the product to the library (bf16, more rows than the
-    weight-streaming kernel takes)."""
+    """Whether ``gemm(a, w, ...)`` hands the product to the library: bf16 with more rows than the
+    weight-streaming kernel takes; or more than one tile of rows over a deep and narrow weight
+    (K >= 2 N), where that kernel has few workgroups and each re-reads every row of ``a`` along
+    a long K (measured at [2048, 8192] and 32 rows: 19 us against the library's 15)."""
     m, k = a.shape
+    n = w.shape[0]
     lda = a.stride(0) if m > 1 else k
-    return (a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0 and m > SKINNY_MAX_M)
+    return (a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0
+            and (m > SKINNY_MAX_M or (m > 16 and k >= 2 * n)))
 
 
 def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -288,7 +297,7 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> Non
     if not accumulate:
         _tcode(out.dtype)
     if a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0:
-        if m <= SKINNY_MAX_M:
+        if not is_library_product(a, w):
             f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
             wp, tiled = _w_args(w)
             _ok(f(a.data_ptr(), 0, wp, tiled, out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
@@ -318,7 +327,7 @@ def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: flo
     ``out: [M, N/2]`` bf16.  Callers check ``bf16_kernel_takes`` first."""
     rms = rms_eps is not None
     m, n, k, lda, ldc = _gemm_operands(a, w, out, (lambda n: n // 2) if silu_pairs else (lambda n: n))
-    if not bf16_kernel_takes(a, w, rms):
+    if not bf16_kernel_takes(a, w, rms, silu_pairs):
         raise KernelError("gemm_fused: operands do not fit the MFMA kernel")
     if silu_pairs:
         if n % 4 or out.dtype != BF16 or accumulate:
@@ -352,7 +361,7 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     m, k = a.shape
     _check(a, "a", None, (m, k), contiguous=False)
     _check(plain_of(w), "w", BF16, ((H + 2 * KV) * d, k))
-    if not bf16_kernel_takes(a, w, rms) or a.stride(1) != 1:
+    if not bf16_kernel_takes(a, w, rms, True) or a.stride(1) != 1:
         raise KernelError("gemm_qkv_rope: operands do not fit the MFMA kernel")
     _check(q_out, "q_out", BF16, (m, H * d))
     _check(positions, "positions", I32, (None,))

@@ -113,7 +113,7 @@ class PagedAttention(Mixer):
             x, rms = normed, None
         else:
             step.settle()
-        if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None) and layer.k_pages.dtype == torch.bfloat16:
+        if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True) and layer.k_pages.dtype == torch.bfloat16:
             # one kernel: (norm,) projection, rotary, cache write
             qkv = ws.buf("q_rot", (n, H * d), act)
             ops.gemm_qkv_rope(x, self.w_qkv, qkv, step.positions, step.seq_of_token, cos, sin, table,

@@ -71,7 +71,7 @@ class SwiGLU(FeedForward):
             x, rms = normed, None
         else:
             step.settle()
-        if ops.bf16_kernel_takes(x, self.w_gate_up, rms is not None) and self.inter % 2 == 0:
+        if ops.bf16_kernel_takes(x, self.w_gate_up, rms is not None, True) and self.inter % 2 == 0:
             # one kernel: (norm,) gate/up projection, SwiGLU gate
             ops.gemm_fused(x, self.w_gate_up, act, rms_eps=rms, silu_pairs=True)
         else:

@@ -111,8 +111,9 @@ def test_gemm_generic(ta, tw, mnk):
     a = torch.randn(m, k, generator=g).to(ta)
     w = (torch.randn(n, k, generator=g) * 0.1).to(tw)
     want = a.double() @ w.double().T
-    # bf16 x bf16 with more than 16 rows goes to the library, whose product is rounded to bf16
-    library = ta == tw == torch.bfloat16 and k % 8 == 0 and m > ops().SKINNY_MAX_M
+    # bf16 x bf16 with many rows goes to the library, whose product is rounded to bf16
+    library = ops().is_library_product(a.to(DEV), w.to(DEV))
+    assert library == (ta == tw == torch.bfloat16 and k % 8 == 0 and m > ops().SKINNY_MAX_M)
     t32 = tol(torch.bfloat16) if library else dict(atol=2e-5, rtol=2e-5)
     for out_dtype in DTYPES:
         out = torch.empty(m, n, dtype=out_dtype, device=DEV)
@@ -140,9 +141,11 @@ def test_gemm_bf16_mfma(m, n, k):
     a = torch.randn(m, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
     want = a.double() @ w.double().T
-    # up to 16 rows the hand-written kernel keeps fp32 sums; beyond, the library's product is
-    # rounded to bf16 before it is widened or added
-    t32 = dict(atol=1e-4, rtol=1e-4) if m <= ops().SKINNY_MAX_M else dict(atol=2e-2, rtol=2e-2)
+    # the hand-written kernel keeps fp32 sums; the library's product is rounded to bf16 before
+    # it is widened or added
+    own = not ops().is_library_product(a.to(DEV), w.to(DEV))
+    assert own == (m <= 16 or (m <= ops().SKINNY_MAX_M and k < 2 * n))
+    t32 = dict(atol=1e-4, rtol=1e-4) if own else dict(atol=2e-2, rtol=2e-2)
     out = torch.empty(m, n, device=DEV)
     ops().gemm(a.to(DEV), w.to(DEV), out)
     torch.testing.assert_close(out.double().cpu(), want, **t32)
@@ -201,7 +204,7 @@ def test_gemm_over_tiled_weights_gives_the_same_bits(m, n, k):
     assert torch.equal(o1, o2)
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 20])
+@pytest.mark.parametrize("m", [1, 8, 16, 20, 33, 50, 64])
 @pytest.mark.parametrize("n,k", [(352, 96), (512, 2048), (48, 40)])
 def test_gemm_fused_norm_and_gate(m, n, k):
     """The MFMA kernel with the RMS norm folded into its left operand (fp32 rows, factor
@@ -229,7 +232,7 @@ def test_gemm_fused_norm_and_gate(m, n, k):
         with pytest.raises(ops().KernelError):
             ops().gemm_fused(x.to(DEV), w.to(DEV), out, rms_eps=eps)
     xb = xn.to(torch.bfloat16)
-    if m <= ops().SKINNY_MAX_M:
+    if m <= ops().FUSED_EPILOGUE_MAX_M:
         ops().gemm_fused(xb.to(DEV), w.to(DEV), gate, silu_pairs=True)
         wantb = xb.double() @ w.double().T
         torch.testing.assert_close(gate.double().cpu(),
@@ -237,7 +240,7 @@ def test_gemm_fused_norm_and_gate(m, n, k):
                                    atol=1e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("m", [1, 9, 16])
+@pytest.mark.parametrize("m", [1, 9, 16, 23, 40, 64])
 @pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16),
                                             (32, 8, 64, 64, 16)])
 @pytest.mark.parametrize("rms", [False, True])
