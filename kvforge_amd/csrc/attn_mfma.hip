@@ -33,10 +33,11 @@
 //   stages are in flight: page lookups two blocks ahead, fragment loads one block ahead
 //   (registers, then the other half of a double LDS buffer), products of this block.
 // Few rows, long key range: a workgroup takes one row tile and one of `splits` cuts of the key
-//   range; its waves (eight, or four where the grid fills the chip) take the blocks of that cut in
-//   turn and are merged through LDS; with
-//   splits > 1 partial (max, sum, accumulator) go to a workspace that
-//   `attn_split_combine_kernel` merges in split order.
+//   range; blocks of 32 keys go round the waves (eight, or four where the grid fills the chip) of
+//   all cuts in turn, so a wave's first block does not depend on the context length and its page
+//   lookups leave with the first loads.  The waves are merged through LDS; with splits > 1
+//   partial (max, sum, accumulator) go to a workspace that `attn_split_combine_kernel` merges in
+//   split order.
 // block_size must be a multiple of 8 (a lane's eight keys lie in one page), d a multiple of 16;
 // kernels are instantiated for each d / 16 so that no loop bound is left to run time.
 #include "common.h"
@@ -492,13 +493,14 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     hi = pos_max < ctx - 1 ? pos_max : ctx - 1;
     if (a.window > 0 && pos_min - a.window + 1 > 0) lo = pos_min - a.window + 1;
   }
+  // Blocks of 32 keys go round the waves of all cuts in turn: cut z, wave w take blocks
+  // z * NW + w, then every (NW * splits)-th.  Without a window the first block is known before
+  // the context length has arrived.
   const int kb0 = (lo / 32) * 32;
-  const int blocks = hi >= kb0 ? (hi - kb0) / 32 + 1 : 0;
-  int per = (blocks + a.splits - 1) / a.splits;
-  per = (per + NW - 1) / NW * NW;  // whole rounds of the waves
-  const int kb_end = min(hi + 1, kb0 + (static_cast<int>(blockIdx.z) + 1) * per * 32);
-  const int kb_begin = kb0 + (blockIdx.z * per + wave) * 32;
-  constexpr int STEP = 32 * NW;
+  const int kb_end = hi + 1;
+  const int turn = (static_cast<int>(blockIdx.z) * NW + wave) * 32;
+  const int kb_begin = kb0 + turn;
+  const int STEP = 32 * NW * a.splits;
   const float scale2 = a.scale * LOG2E;
 
   float m_ref[1] = {-INFINITY}, l_run[1] = {0.f};
@@ -538,12 +540,21 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
     block_update<DT, 1>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
   };
+  // Without a window the page lookups of the first blocks are asked for together with the
+  // query and the context length, not after them: one round trip to memory less.
+  const bool early = a.window <= 0;
+  if (early) {
+    locate(turn, pA);
+    if (TWO) locate(turn + STEP, pB);
+  }
   // the query fragments have to be there before the loops (see the note in the runs kernel)
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   if (TWO) {
     if (kb_begin < kb_end) {
-      locate(kb_begin, pA);
-      locate(kb_begin + STEP, pB);
+      if (!early) {
+        locate(kb_begin, pA);
+        locate(kb_begin + STEP, pB);
+      }
       fetch(kb_begin, pA, A);
     }
     for (int kb = kb_begin; kb < kb_end; kb += 2 * STEP) {
@@ -558,7 +569,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
       }
     }
   } else {
-    locate(kb_begin, pA);
+    if (!early) locate(kb_begin, pA);
     for (int kb = kb_begin; kb < kb_end; kb += STEP) {
       fetch(kb, pA, A);
       locate(kb + STEP, pA);
