@@ -303,11 +303,152 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
   }
 }
 
+// The same work for a tile of 16 tokens per workgroup with 8 elements per lane and access
+// (d and the rotary width multiples of 8).  V is stored transposed, so a token's elements lie
+// block_size apart; where the tile's 16 tokens fill consecutive places of one page (a prompt
+// read from a page boundary) the tile is turned in LDS and each (head, element) row of 16
+// tokens is stored in one piece.  Other tiles store V element by element.
+constexpr int ROPE_TILE = 16;
+
+__device__ __forceinline__ void store8(float* p, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+__device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = static_cast<uint32_t>(f32_to_bf16(v[2 * i])) | (static_cast<uint32_t>(f32_to_bf16(v[2 * i + 1])) << 16);
+  *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kvwrite_tile_kernel(
+    T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ block_table, T* __restrict__ k_pages, T* __restrict__ v_pages, int n,
+    int turn_v, RopeArgs a) {
+  extern __shared__ __align__(16) unsigned char tile_raw[];  // [ROPE_TILE][V columns of this share] of T, if turn_v
+  __shared__ int s_pos[ROPE_TILE], s_page[ROPE_TILE], s_off[ROPE_TILE], s_run;
+  const int n0 = blockIdx.x * ROPE_TILE;
+  const int cnt = min(ROPE_TILE, n - n0);
+  const int half = a.rot / 2;
+  if (threadIdx.x < ROPE_TILE) {
+    const int t = threadIdx.x;
+    int p = -1, page = -1, off = 0;
+    if (t < cnt) {
+      p = positions[n0 + t];
+      if (p < 0 || p >= a.table_len) p = -1;
+      if (p >= 0 && a.write_kv) {
+        const int seq = seq_of_token[n0 + t];
+        const int blk = p / a.block_size;
+        if (seq >= 0 && seq < a.n_seqs && blk < a.table_stride) {
+          page = block_table[static_cast<size_t>(seq) * a.table_stride + blk];
+          if (page >= a.num_blocks) page = -1;
+          off = p - blk * a.block_size;
+        }
+      }
+    }
+    s_pos[t] = p;
+    s_page[t] = page;
+    s_off[t] = off;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    bool run = turn_v && cnt == ROPE_TILE && s_page[0] >= 0 && s_off[0] % 8 == 0 &&
+               a.block_size % 8 == 0 && s_off[0] + ROPE_TILE <= a.block_size;
+    for (int t = 1; t < ROPE_TILE; ++t) run = run && s_page[t] == s_page[0] && s_off[t] == s_off[0] + t;
+    s_run = run;
+  }
+  __syncthreads();
+  // blockIdx.y names a share of the row: of its q and k vectors, and of its V columns
+  const int row_len = (a.H + 2 * a.KV) * a.d;
+  const int qk_vecs = (a.H + a.KV) * a.d / 8;
+  const int qk_share = (qk_vecs + gridDim.y - 1) / gridDim.y;
+  const int qk_begin = blockIdx.y * qk_share;
+  const int qk_mine = max(0, min(qk_share, qk_vecs - qk_begin));
+  for (int item = threadIdx.x; item < cnt * qk_mine; item += blockDim.x) {
+    const int t = item / qk_mine, e = (qk_begin + item - t * qk_mine) * 8;
+    const int head = e / a.d, i0 = e - head * a.d;
+    const bool is_k = head >= a.H;
+    const int p = s_pos[t], page = s_page[t];
+    // a query that is not rotated stays as it is; a key without a page is not stored
+    if (is_k ? page < 0 : (p < 0 || i0 >= a.rot)) continue;
+    T* src = qkv + static_cast<size_t>(n0 + t) * row_len + e;
+    float x[8];
+    load8(src, x);
+    if (p >= 0 && i0 < a.rot) {
+      const float4 c = *reinterpret_cast<const float4*>(cos_t + static_cast<size_t>(p) * half + i0 / 2);
+      const float4 sn = *reinterpret_cast<const float4*>(sin_t + static_cast<size_t>(p) * half + i0 / 2);
+      const float cs[4] = {c.x, c.y, c.z, c.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float x1 = x[2 * i], x2 = x[2 * i + 1];
+        x[2 * i] = x1 * cs[i] - x2 * ss[i];
+        x[2 * i + 1] = x2 * cs[i] + x1 * ss[i];
+      }
+    }
+    T* dst = is_k ? k_pages + ((static_cast<size_t>(page) * a.KV + (head - a.H)) * a.block_size + s_off[t]) * a.d + i0
+                  : src;
+    store8(dst, x);
+  }
+  if (!a.write_kv) return;
+  const int v0 = (a.H + a.KV) * a.d, v_len = a.KV * a.d;
+  const int v_share = (v_len / 8 + gridDim.y - 1) / gridDim.y * 8;  // columns, whole vectors
+  const int v_begin = blockIdx.y * v_share;
+  const int v_mine = max(0, min(v_share, v_len - v_begin));
+  if (s_run) {
+    T* tile = reinterpret_cast<T*>(tile_raw);  // [ROPE_TILE][v_share]
+    const int v_vecs = v_mine / 8;
+    for (int item = threadIdx.x; item < ROPE_TILE * v_vecs; item += blockDim.x) {
+      const int t = item / v_vecs, e = (item - t * v_vecs) * 8;
+      const T* src = qkv + static_cast<size_t>(n0 + t) * row_len + v0 + v_begin + e;
+      constexpr int Q = sizeof(T) * 8 / 16;  // 16-byte pieces of eight elements
+#pragma unroll
+      for (int q = 0; q < Q; ++q)
+        reinterpret_cast<uint4*>(tile + t * v_share + e)[q] = reinterpret_cast<const uint4*>(src)[q];
+    }
+    __syncthreads();
+    const int page = s_page[0], off0 = s_off[0];
+    for (int c = threadIdx.x; c < v_mine; c += blockDim.x) {  // v_begin + c = head * d + element
+      __align__(16) T vals[ROPE_TILE];
+#pragma unroll
+      for (int t = 0; t < ROPE_TILE; ++t) vals[t] = tile[t * v_share + c];
+      T* dst = v_pages + (static_cast<size_t>(page) * v_len + v_begin + c) * a.block_size + off0;
+      constexpr int Q = sizeof(T) * ROPE_TILE / 16;
+#pragma unroll
+      for (int q = 0; q < Q; ++q) reinterpret_cast<uint4*>(dst)[q] = reinterpret_cast<const uint4*>(vals)[q];
+    }
+  } else {
+    for (int item = threadIdx.x; item < cnt * v_mine; item += blockDim.x) {
+      const int t = item / v_mine, c = v_begin + item - t * v_mine;
+      const int page = s_page[t];
+      if (page < 0) continue;
+      v_pages[(static_cast<size_t>(page) * v_len + c) * a.block_size + s_off[t]] =
+          qkv[static_cast<size_t>(n0 + t) * row_len + v0 + c];
+    }
+  }
+}
+
 template <typename T>
 static int rope_launch(void* qkv, const int* positions, const int* seq_of_token, const float* cos_t,
                        const float* sin_t, const int* block_table, void* k_pages, void* v_pages,
                        int n, RopeArgs a, hipStream_t s) {
   if (n <= 0) return 0;
+  if (a.d % 8 == 0 && a.rot % 8 == 0) {
+    // few tiles: several workgroups share a tile's row, so that the chip has work
+    const int tiles = (n + ROPE_TILE - 1) / ROPE_TILE;
+    int shares = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
+    if (shares > 8) shares = 8;
+    const int v_share = (a.KV * a.d / 8 + shares - 1) / shares * 8;
+    // the tile of V rows turned in LDS; without room for it V goes element by element
+    const size_t lds = static_cast<size_t>(ROPE_TILE) * v_share * sizeof(T);
+    const int turn_v = lds <= 48 * 1024;
+    hipLaunchKernelGGL(rope_kvwrite_tile_kernel<T>, dim3(tiles, shares), dim3(256), turn_v ? lds : 0, s,
+                       static_cast<T*>(qkv), positions, seq_of_token, cos_t, sin_t, block_table,
+                       static_cast<T*>(k_pages), static_cast<T*>(v_pages), n, turn_v, a);
+    return kvf_last_error();
+  }
   hipLaunchKernelGGL(rope_kvwrite_kernel<T>, dim3(n), dim3(128), 0, s, static_cast<T*>(qkv),
                      positions, seq_of_token, cos_t, sin_t, block_table, static_cast<T*>(k_pages),
                      static_cast<T*>(v_pages), a);

@@ -542,18 +542,35 @@ def test_attn_far_key_stands_out():
         torch.testing.assert_close(out.cpu(), want, atol=2e-5, rtol=2e-5)
 
 
+# (sequence, first position, tokens) of each portion in the flat batch.  The kernel takes the
+# batch in tiles of 16 tokens and writes V by whole runs where a tile lies in one page: the cases
+# hold tiles that do (pages of 16 from position 0 or 16, pages of 32 from position 8), tiles that
+# straddle pages or sequences, a short last tile, and a page that was given back.
+ROPE_BATCHES = {
+    "mixed": [(0, 2, 5), (1, 0, 19)],              # the first sequence already holds two tokens
+    "aligned": [(1, 0, 37)],
+    "offset": [(0, 8, 16), (1, 16, 20)],
+    "late_start": [(0, 0, 3), (1, 3, 34)],
+}
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16)])
-def test_rope_kvwrite(dtype, H, KV, d, rot, bs):
+@pytest.mark.parametrize("batch", sorted(ROPE_BATCHES))
+@pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16),
+                                            (5, 2, 20, 12, 16), (2, 1, 64, 64, 32), (8, 8, 128, 128, 16)])
+def test_rope_kvwrite(dtype, batch, H, KV, d, rot, bs):
     g = torch.Generator().manual_seed(d)
-    seq_lens = [5, 19]
-    starts = [2, 0]                      # the first sequence already holds two tokens
-    n = sum(seq_lens)
+    portions = ROPE_BATCHES[batch]
+    n = sum(c for _, _, c in portions)
     qkv = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
-    positions = torch.tensor([starts[0] + i for i in range(5)] + list(range(19)), dtype=torch.int32)
-    seq_of = torch.tensor([0] * 5 + [1] * 19, dtype=torch.int32)
-    nb = 12
-    table = torch.tensor([[7, 3, -1, -1, -1], [1, 9, 4, 0, 2]], dtype=torch.int32)[:, : -(-21 // bs) + 1]
+    positions = torch.tensor([p0 + i for _, p0, c in portions for i in range(c)], dtype=torch.int32)
+    seq_of = torch.tensor([sq for sq, _, c in portions for _ in range(c)], dtype=torch.int32)
+    nb = 24
+    width = -(-40 // bs) + 1
+    table = torch.randperm(nb, generator=g)[:2 * width].reshape(2, width).to(torch.int32)
+    table[0, -(-24 // bs):] = -1                   # the first sequence has no pages past 24 tokens
+    if batch == "mixed":
+        table[1, 0] = -1                           # a page that was given back
     table = table.contiguous()
     inv_freq = plain.rope_inv_freq(rot, 10000.0)
     cos_full, sin_full = plain.rope_cos_sin(torch.arange(40), inv_freq)
