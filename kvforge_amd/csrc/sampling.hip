@@ -1,4 +1,4 @@
-// Token selection from fp32 logits, one workgroup of 16 waves per row.
+// Token selection from fp32 logits, one workgroup of 16 waves per row (several for greedy rows).
 //
 //   temperature == 0      : argmax, the lowest index among equal maxima.
 //   temperature  > 0      : z = logits / temperature; optional top-k, then optional top-p on the
@@ -40,11 +40,18 @@ __device__ __forceinline__ float block_reduce_max(float v, float* sh) {
   return t;
 }
 
+// Greedy rows may be cut into `splits` chunks, one workgroup each (blockIdx.y): a row of a large
+// vocabulary is then read by several compute units.  Every workgroup leaves the best of its chunk
+// in `work` and takes a ticket; the one that takes the row's last ticket picks the best of the
+// chunks in chunk order (so equal maxima still give the lowest index) and puts the tickets back
+// to zero.  Nobody waits for anybody.  `work` (int32): [rows] tickets, zero before the first
+// launch; [rows * splits] values; [rows * splits] indices.  Rows that sample are done by the
+// workgroup of chunk 0 alone.
 __global__ __launch_bounds__(THREADS) void sample_kernel(
     const float* __restrict__ logits, int ld, int V, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ u,
     const int* __restrict__ u_step, int u_stride,
-    int* __restrict__ tokens) {
+    int* __restrict__ tokens, int* __restrict__ work) {
   __shared__ float sh[NWAVES];
   __shared__ float seg_sum[NWAVES];
   __shared__ int sh_idx[NWAVES];
@@ -55,17 +62,21 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
   const float temp = temperature[row];
 
   if (!(temp > 0.f)) {  // greedy
+    const int splits = gridDim.y, rows = gridDim.x;
+    // chunks of whole groups of four elements
+    const int chunk = ((V + splits - 1) / splits + 3) & ~3;
+    const int lo = min(V, static_cast<int>(blockIdx.y) * chunk), hi = min(V, lo + chunk);
     float best = -INFINITY;
     int bi = V;
     // rows of 4 floats at a time where the row is 16-byte aligned; several loads in flight
     const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-    const int v4 = vec ? V / 4 : 0;
+    const int a4 = lo / 4, b4 = vec ? hi / 4 : a4;
     const float4* x4 = reinterpret_cast<const float4*>(x);
-    for (int i0 = tid; i0 < v4; i0 += 4 * THREADS) {
+    for (int i0 = a4 + tid; i0 < b4; i0 += 4 * THREADS) {
       float4 r[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        r[u] = i0 + u * THREADS < v4 ? x4[i0 + u * THREADS] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        r[u] = i0 + u * THREADS < b4 ? x4[i0 + u * THREADS] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const int base = 4 * (i0 + u * THREADS);
@@ -75,7 +86,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
           if (e[c] > best || (e[c] == best && base + c < bi)) { best = e[c]; bi = base + c; }
       }
     }
-    for (int i = 4 * v4 + tid; i < V; i += THREADS) {
+    for (int i = 4 * b4 + tid; i < hi; i += THREADS) {
       const float v = x[i];
       if (v > best || (v == best && i < bi)) { best = v; bi = i; }
     }
@@ -89,10 +100,34 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
     if (tid == 0) {
       for (int w = 1; w < NWAVES; ++w)
         if (sh[w] > best || (sh[w] == best && sh_idx[w] < bi)) { best = sh[w]; bi = sh_idx[w]; }
-      tokens[row] = bi < V ? bi : 0;
+      if (splits == 1) {
+        tokens[row] = bi < V ? bi : 0;
+      } else {
+        int* vals = work + rows;
+        int* idxs = vals + rows * splits;
+        const int slot = row * splits + blockIdx.y;
+        __hip_atomic_store(vals + slot, __float_as_int(best), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(idxs + slot, bi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();  // the chunk's best is visible to the device before the ticket is taken
+        const int ticket = atomicAdd(work + row, 1);
+        if (ticket == splits - 1) {
+          __threadfence();
+          best = -INFINITY;
+          bi = V;
+          for (int c = 0; c < splits; ++c) {
+            const float v = __int_as_float(
+                __hip_atomic_load(vals + row * splits + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            const int i = __hip_atomic_load(idxs + row * splits + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (v > best || (v == best && i < bi)) { best = v; bi = i; }
+          }
+          tokens[row] = bi < V ? bi : 0;
+          __hip_atomic_store(work + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
     }
     return;
   }
+  if (blockIdx.y != 0) return;
 
   const float inv_t = 1.f / temp;
   float mx = -INFINITY;
@@ -215,13 +250,17 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(
 
 // u_step (may be null): a device counter; row r then draws with u[*u_step * u_stride + r], so
 // that a captured launch can be replayed for several decode steps, each with numbers of its own.
+// work (may be null) with splits > 1: greedy rows are read by `splits` workgroups each; it holds
+// rows * (1 + 2 * splits) int32, the first `rows` of them zero, and is left so.  Launches that
+// share it must not overlap.
 KVF_EXPORT int kvf_sample(const float* logits, int ld, int rows, int V, const float* temperature,
                           const int* top_k, const float* top_p, const float* u, const int* u_step,
-                          int u_stride, int* tokens, hipStream_t s) {
+                          int u_stride, int* tokens, int* work, int splits, hipStream_t s) {
   if (rows <= 0) return 0;
-  if (V <= 0 || ld < V) return static_cast<int>(hipErrorInvalidValue);
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(THREADS), 0, s, logits, ld, V, temperature,
-                     top_k, top_p, u, u_step, u_stride, tokens);
+  if (V <= 0 || ld < V || splits < 1 || splits > 64 || (splits > 1 && !work))
+    return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(sample_kernel, dim3(rows, splits), dim3(THREADS), 0, s, logits, ld, V, temperature,
+                     top_k, top_p, u, u_step, u_stride, tokens, work);
   return kvf_last_error();
 }
 

@@ -65,6 +65,8 @@ class ModelRunner:
         self._sample_f = torch.zeros(nf, dtype=torch.float32, device=self.device)
         self._sample_i = torch.zeros(2 * cap, dtype=torch.int32, device=self.device)
         self._run_counter = torch.zeros(1, dtype=torch.int32, device=self.device)
+        # tickets and chunk results of greedy rows read by several workgroups (zero between launches)
+        self._sample_work = torch.zeros(ops.sample_work_size(cap), dtype=torch.int32, device=self.device)
         self._run_ring = torch.zeros(MAX_DECODE_RUN, cap, dtype=torch.int32, device=self.device)
         self._sample_f_host = torch.zeros(nf, dtype=torch.float32, pin_memory=True)
         self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
@@ -192,7 +194,7 @@ class ModelRunner:
         sampled = self._sample_i[cap:cap + rows]
         ops.sample(logits, self._sample_f[:rows], self._sample_i[:rows],
                    self._sample_f[cap:cap + rows], self._sample_f[2 * cap:].view(MAX_DECODE_RUN, cap),
-                   sampled, self._run_counter)
+                   sampled, self._run_counter, self._sample_work)
         ops.decode_advance(sampled, step.token_ids, step.positions, step.ctx_lens, self._run_ring,
                            self._run_counter)
         return logits

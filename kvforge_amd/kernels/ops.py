@@ -524,13 +524,25 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
 
 
 # ------------------------------------------------------------------------------ sampling
+GREEDY_SPLIT_MAX = 16
+
+
+def sample_work_size(rows: int) -> int:
+    """int32 elements of the ``work`` tensor that lets ``sample`` read greedy rows with several
+    workgroups each: tickets, then the best value and index of every chunk."""
+    return rows * (1 + 2 * GREEDY_SPLIT_MAX)
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor | None,
            top_p: torch.Tensor | None, u: torch.Tensor, tokens: torch.Tensor,
-           u_step: torch.Tensor | None = None) -> None:
+           u_step: torch.Tensor | None = None, work: torch.Tensor | None = None) -> None:
     """One token per row of fp32 ``logits``: argmax where ``temperature == 0``, otherwise the
     inverse CDF of the processed distribution at ``u``.  With ``u_step`` (one int32 on the
     device) ``u`` holds several rows of numbers, ``[steps, row stride]``, and row ``u_step[0]``
-    is used: a captured launch then serves several decode steps."""
+    is used: a captured launch then serves several decode steps.  ``work`` (int32,
+    ``sample_work_size(rows)`` elements, zero when first handed over, not shared with a launch
+    that may overlap): greedy rows are then read by several workgroups each, about as many as
+    fill the chip; the result is the same."""
     _check(logits, "logits", F32, (None, None), contiguous=False)
     if logits.stride(1) != 1:
         raise KernelError("sample: logits rows must be dense")
@@ -550,13 +562,21 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor 
         _check(top_k, "top_k", I32, (r,))
     if top_p is not None:
         _check(top_p, "top_p", F32, (r,))
+    splits = 1
+    if work is not None:
+        _check(work, "work", I32, (None,))
+        if work.shape[0] < sample_work_size(r):
+            raise KernelError("sample: work is smaller than sample_work_size(rows)")
+        # about one workgroup per compute unit, each with at least 4096 logits
+        splits = max(1, min(GREEDY_SPLIT_MAX, 256 // r, v // 4096))
     f = _fn("sampling", "kvf_sample",
-            [c_void_p, c_int, c_int, c_int] + [c_void_p] * 5 + [c_int, c_void_p, c_void_p])
+            [c_void_p, c_int, c_int, c_int] + [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int,
+                                                                c_void_p])
     _ok(f(logits.data_ptr(), logits.stride(0) if r > 1 else v, r, v, temperature.data_ptr(),
           top_k.data_ptr() if top_k is not None else None,
           top_p.data_ptr() if top_p is not None else None, u.data_ptr(),
           u_step.data_ptr() if u_step is not None else None, stride, tokens.data_ptr(),
-          _stream()), "sample")
+          work.data_ptr() if work is not None else None, splits, _stream()), "sample")
 
 
 def decode_advance(sampled: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,

@@ -660,6 +660,38 @@ def test_sample_matches_plain(V):
         assert plain_sampling.draw_margin(probs, us[r], got[r]) < 1e-5, f"row {r}"
 
 
+@pytest.mark.parametrize("rows", [1, 8, 37])
+@pytest.mark.parametrize("V", [4100, 50001, 128256])
+def test_sample_greedy_rows_read_in_chunks(rows, V):
+    """Greedy rows cut over several workgroups give the token of one workgroup per row: the
+    largest logit, the lowest index among equal ones (put into different chunks here), also on a
+    second call that finds the tickets of the first; sampled rows beside them are untouched by
+    the cut."""
+    g = torch.Generator().manual_seed(rows * V)
+    wide = torch.randn(rows, V + 3, generator=g)
+    logits = wide[:, :V]                           # an odd vocabulary leaves rows unaligned
+    top = float(logits.max()) + 1.0
+    for r in range(rows):
+        where = torch.randint(0, V, (3,), generator=g)
+        logits[r, where] = top + r                 # the same maximum at up to three places
+    temps = torch.tensor([0.9 if r % 5 == 3 else 0.0 for r in range(rows)])
+    us = torch.tensor([plain_sampling.uniform(1, r, 0) for r in range(rows)])
+    dev_logits = wide.to(DEV)[:, :V]
+    one = torch.empty(rows, dtype=torch.int32, device=DEV)
+    ops().sample(dev_logits, temps.to(DEV), None, None, us.to(DEV), one)
+    work = torch.zeros(ops().sample_work_size(rows), dtype=torch.int32, device=DEV)
+    for _ in range(2):
+        cut = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        ops().sample(dev_logits, temps.to(DEV), None, None, us.to(DEV), cut, work=work)
+        assert torch.equal(cut, one)
+        assert int(work[:rows].abs().sum()) == 0
+    for r in range(rows):
+        if temps[r] == 0.0:
+            assert int(one[r]) == int((logits[r] == logits[r].max()).nonzero()[0])
+    with pytest.raises(ops().KernelError):
+        ops().sample(dev_logits, temps.to(DEV), None, None, us.to(DEV), one, work=work[:rows])
+
+
 def test_sample_frequencies_follow_softmax():
     logits = torch.tensor([1.0, 0.0, -1.0, 2.0, 0.5])
     n = 4000
