@@ -54,9 +54,9 @@ __device__ __forceinline__ void store4(bf16_t* p, const float4& v) {
 
 constexpr int NORM_KEEP = 4;  // float4s a thread keeps in registers between the two passes
 
-template <typename T, typename W>
+template <typename T, typename W, typename D>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ rows,
-                               const T* __restrict__ delta, const W* __restrict__ w, float eps,
+                               const D* __restrict__ delta, const W* __restrict__ w, float eps,
                                T* __restrict__ out, int h, int x_rows, int aligned) {
   __shared__ float scratch[16];
   const int m = blockIdx.x;
@@ -67,7 +67,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ ro
     return;
   }
   float* xr = x + static_cast<size_t>(src) * h;
-  const T* dr = delta ? delta + static_cast<size_t>(src) * h : nullptr;
+  const D* dr = delta ? delta + static_cast<size_t>(src) * h : nullptr;
   const bool write_back = dr && !rows;
   float ss = 0.f;
   if (aligned && h <= static_cast<int>(blockDim.x) * 4 * NORM_KEEP) {
@@ -106,7 +106,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ ro
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
     float v = xr[i];
     if (dr) {
-      v += Elem<T>::load(dr + i);
+      v += Elem<D>::load(dr + i);
       if (write_back) xr[i] = v;
     }
     ss += v * v;
@@ -115,36 +115,39 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const int* __restrict__ ro
   const float r = rsqrtf(ss / static_cast<float>(h) + eps);
   for (int i = threadIdx.x; i < h; i += blockDim.x) {
     float v = xr[i];  // already the sum where it was written back (by this same thread)
-    if (dr && !write_back) v += Elem<T>::load(dr + i);
+    if (dr && !write_back) v += Elem<D>::load(dr + i);
     Elem<T>::store(o + i, w ? v * r * Elem<W>::load(w + i) : v * r);
   }
 }
 
-template <typename T>
+template <typename T, typename D>
 static int rmsnorm_launch(float* x, const int* rows, const void* delta, const void* w, int w_is_f32,
                           float eps, void* out, int m, int h, int x_rows, hipStream_t s) {
   if (m <= 0) return 0;
   const int threads = h >= 1024 ? 256 : (h >= 256 ? 128 : 64);
   auto at = [](const void* p, size_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; };
-  const int aligned = h % 4 == 0 && at(x, 16) && at(out, 4 * sizeof(T)) && at(delta, 4 * sizeof(T)) &&
+  const int aligned = h % 4 == 0 && at(x, 16) && at(out, 4 * sizeof(T)) && at(delta, 4 * sizeof(D)) &&
                       at(w, w_is_f32 ? 16 : 4 * sizeof(T));
   if (w_is_f32)
-    hipLaunchKernelGGL((rmsnorm_kernel<T, float>), dim3(m), dim3(threads), 0, s, x, rows,
-                       static_cast<const T*>(delta), static_cast<const float*>(w), eps,
+    hipLaunchKernelGGL((rmsnorm_kernel<T, float, D>), dim3(m), dim3(threads), 0, s, x, rows,
+                       static_cast<const D*>(delta), static_cast<const float*>(w), eps,
                        static_cast<T*>(out), h, x_rows, aligned);
   else
-    hipLaunchKernelGGL((rmsnorm_kernel<T, T>), dim3(m), dim3(threads), 0, s, x, rows,
-                       static_cast<const T*>(delta), static_cast<const T*>(w), eps,
+    hipLaunchKernelGGL((rmsnorm_kernel<T, T, D>), dim3(m), dim3(threads), 0, s, x, rows,
+                       static_cast<const D*>(delta), static_cast<const T*>(w), eps,
                        static_cast<T*>(out), h, x_rows, aligned);
   return kvf_last_error();
 }
-KVF_EXPORT int kvf_rmsnorm_f32(float* x, const int* rows, const void* delta, const void* w, int wf,
-                               float eps, void* out, int m, int h, int xr, hipStream_t s) {
-  return rmsnorm_launch<float>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
+// delta (may be null): a sum still owed to x, in the type of `out` or (delta_f32) in fp32
+KVF_EXPORT int kvf_rmsnorm_f32(float* x, const int* rows, const void* delta, int delta_f32, const void* w,
+                               int wf, float eps, void* out, int m, int h, int xr, hipStream_t s) {
+  (void)delta_f32;
+  return rmsnorm_launch<float, float>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
 }
-KVF_EXPORT int kvf_rmsnorm_bf16(float* x, const int* rows, const void* delta, const void* w, int wf,
-                                float eps, void* out, int m, int h, int xr, hipStream_t s) {
-  return rmsnorm_launch<bf16_t>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
+KVF_EXPORT int kvf_rmsnorm_bf16(float* x, const int* rows, const void* delta, int delta_f32, const void* w,
+                                int wf, float eps, void* out, int m, int h, int xr, hipStream_t s) {
+  if (delta_f32) return rmsnorm_launch<bf16_t, float>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
+  return rmsnorm_launch<bf16_t, bf16_t>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
 }
 
 // ----------------------------------------------------------------------------- residual sum

@@ -26,6 +26,12 @@
 //   transposed [nb, KV, d, block]).
 // K must be a multiple of 8 (16-byte loads); a k-step that passes K loads zeros.
 //
+// A product that is added to a narrow C over a long K (the down projection) has fewer workgroups
+// than the chip has compute units, and a compute unit keeps only so many bytes in flight.  It
+// may be cut into two halves of K (`Riders::half_out`): a second layer of workgroups stores its
+// half beside C, and the caller owes that half to C.  The next consumers add it on their way:
+// the fused q/k/v projection in its loads (`a_add`), the output projection in its sum (`c_add`).
+//
 // Layout of W.  In the checkpoint's row-major [N, K] a wave's load of one operand fragment
 // touches 16 rows, 64 bytes each: 16 cache lines per group of 16 lanes, and the L1 looks lines up
 // one at a time, which bounds the kernel far below what HBM delivers.  The engine therefore also
@@ -50,22 +56,41 @@ struct RopeEpi {
   int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
 };
 
+// Sums that ride along.  `a_add` (kernels built with ADD): the left operand is A + a_add, both
+// fp32 with the same row stride.  `c_add` (with EPI 2): C += product + c_add, same row stride as C.
+// `half_out` (with EPI 2): the grid is two deep; workgroups of the second layer walk the second
+// half of K and store their product there (fp32, row stride of C) instead of adding it to C, so
+// that a narrow C still puts a workgroup on every compute unit; the caller owes half_out to C.
+struct Riders {
+  const float* a_add;
+  const float* c_add;
+  float* half_out;
+};
+
 __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
   uint4 r = make_uint4(0u, 0u, 0u, 0u);
   if (ok) r = *reinterpret_cast<const uint4*>(p);
   return __builtin_bit_cast(bf16x8, r);
 }
 
-// 8 fp32 -> 8 bf16 (round to nearest even); adds their squares to ss
-__device__ __forceinline__ bf16x8 load_frag_f32(const float* p, bool ok, float& ss) {
+// 8 fp32 (with ADD plus 8 of `q`) -> 8 bf16 (round to nearest even); adds their squares to ss.
+// Nothing inside the branches uses what they load, so no branch ends in a wait and the loads of
+// a whole pass stay in flight together.
+template <bool ADD>
+__device__ __forceinline__ bf16x8 load_frag_f32(const float* p, const float* q, bool ok, float& ss) {
   typedef __attribute__((ext_vector_type(8))) float f32x8;
   float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  if (ok) load8(p, v);
+  float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (ok) {
+    load8(p, v);
+    if (ADD) load8(q, w);
+  }
   f32x8 x;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    ss = fmaf(v[i], v[i], ss);
-    x[i] = v[i];
+    const float t = ADD ? v[i] + w[i] : v[i];
+    ss = fmaf(t, t, ss);
+    x[i] = t;
   }
   return __builtin_convertvector(x, bf16x8);
 }
@@ -90,15 +115,17 @@ __device__ __forceinline__ bool vec4_ok(const void* Cv, int ldc, int n, int N, i
 // First stage: loads that need only (m, n).
 template <int EPI>
 __device__ __forceinline__ void epi_prefetch_a(EpiOperands& op, int m, int n, int N, int ldc, const void* Cv,
-                                               const RopeEpi& rp) {
+                                               const float* c_add, const RopeEpi& rp) {
   op.have = true;
   if (EPI == 2) {
-    const float* c = static_cast<const float*>(Cv) + static_cast<size_t>(m) * ldc + n;
-    if (vec4_ok(Cv, ldc, n, N, 4)) {
+    const size_t idx = static_cast<size_t>(m) * ldc + n;
+    const float* c = static_cast<const float*>(Cv) + idx;
+    if (vec4_ok(Cv, ldc, n, N, 4) && vec4_ok(c_add, ldc, n, N, 4)) {
       op.c = *reinterpret_cast<const f32x4*>(c);
+      if (c_add) op.c += *reinterpret_cast<const f32x4*>(c_add + idx);
     } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) op.c[r] = n + r < N ? c[r] : 0.f;
+      for (int r = 0; r < 4; ++r) op.c[r] = n + r < N ? c[r] + (c_add ? c_add[idx + r] : 0.f) : 0.f;
     }
   }
   if (EPI == 4) {
@@ -133,10 +160,10 @@ __device__ __forceinline__ void epi_prefetch_b(EpiOperands& op, int n, const Rop
 // One lane's four neighbouring columns n..n+3 of row m, after the waves' partial sums are added.
 template <int EPI>
 __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, int ldc, void* Cv,
-                                           const RopeEpi& rp, EpiOperands& op) {
+                                           const float* c_add, const RopeEpi& rp, EpiOperands& op) {
   if (EPI == 2 || EPI == 4) {
     if (!op.have) {
-      epi_prefetch_a<EPI>(op, m, n, N, ldc, Cv, rp);
+      epi_prefetch_a<EPI>(op, m, n, N, ldc, Cv, c_add, rp);
       epi_prefetch_b<EPI>(op, n, rp);
     }
   }
@@ -211,10 +238,10 @@ constexpr int depth(int mt, int nt, int at) {
   return at ? (mt == 1 ? 4 : mt <= 4 ? 2 : 1) : (mt * nt == 1 ? 8 : mt * nt <= 4 ? 4 : 2);
 }
 
-template <int MT, int NT, int AT, int EPI>
+template <int MT, int NT, int AT, int EPI, bool ADD>
 __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
-    int K, int lda, int ldc, int m_base, float eps, int w_tiled, RopeEpi rp) {
+    int K, int lda, int ldc, int m_base, float eps, int w_tiled, Riders rd, RopeEpi rp) {
   constexpr int RW = 16;  // rows of W per group
   extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
@@ -222,6 +249,11 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
   const int n0 = blockIdx.x * RW * NT;
   const int r16 = lane % 16, kg = lane / 16;
   const int ksteps = (K + 31) / 32;
+  // the k-steps this workgroup walks: all, or one half of them (see Riders::half_out)
+  const bool halves = EPI == 2 && rd.half_out != nullptr;
+  const bool second = halves && blockIdx.y == 1;
+  const int ks_cut = halves ? (ksteps + 1) / 2 : ksteps;
+  const int ks_lo = second ? ks_cut : 0, ks_hi = second ? ksteps : ks_cut;
   // where this lane's fragment of k-step 0 lies, and how far the next k-step is
   const bf16_t* wp[NT];
   const size_t w_step = w_tiled ? KVF_WAVE * 8 : 32;
@@ -248,6 +280,8 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
   }
   const bf16_t* Ab = static_cast<const bf16_t*>(Av);
   const float* Af = static_cast<const float*>(Av);
+  const float* a_add = ADD ? rd.a_add : nullptr;
+  const float* c_add = EPI == 2 && !second ? rd.c_add : nullptr;
   f32x4 acc[NT][MT];
   float ss[MT];
 #pragma unroll
@@ -264,17 +298,17 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
 #pragma unroll
   for (int j = 0; j < NT; ++j) pre[j].have = false;
   const int pre_m = m_base + r16, pre_n = n0 + 4 * kg;
-  const bool pre_mine = PRE && wave == 0 && pre_m < M;
+  const bool pre_mine = PRE && wave == 0 && pre_m < M && !second;
   if (pre_mine) {
 #pragma unroll
     for (int j = 0; j < NT; ++j)
-      if (pre_n + j * RW < N) epi_prefetch_a<EPI>(pre[j], pre_m, pre_n + j * RW, N, ldc, Cv, rp);
+      if (pre_n + j * RW < N) epi_prefetch_a<EPI>(pre[j], pre_m, pre_n + j * RW, N, ldc, Cv, c_add, rp);
   }
 
   constexpr int U = depth(MT, NT, AT);
-  int ks = wave;
+  int ks = ks_lo + wave;
   bool first = true;
-  for (; ks + (U - 1) * nw < ksteps; ks += U * nw) {
+  for (; ks + (U - 1) * nw < ks_hi; ks += U * nw) {
     bf16x8 wf[U][NT], af[U][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -284,7 +318,7 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       for (int j = 0; j < NT; ++j) wf[u][j] = load_frag(wp[j] + (ks + u * nw) * w_step, ok || w_tiled);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        af[u][t] = AT ? load_frag_f32(Af + aoff[t] + k, ok && a_live[t], ss[t])
+        af[u][t] = AT ? load_frag_f32<ADD>(Af + aoff[t] + k, a_add + aoff[t] + k, ok && a_live[t], ss[t])
                       : load_frag(Ab + aoff[t] + k, ok && a_live[t]);
     }
 #pragma unroll
@@ -308,13 +342,13 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
     for (int j = 0; j < NT; ++j)
       if (pre[j].have) epi_prefetch_b<EPI>(pre[j], pre_n + j * RW, rp);
   }
-  for (; ks < ksteps; ks += nw) {
+  for (; ks < ks_hi; ks += nw) {
     const int k = ks * 32;
     const bool ok = k + kg * 8 + 8 <= K;
     bf16x8 af[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t)
-      af[t] = AT ? load_frag_f32(Af + aoff[t] + k, ok && a_live[t], ss[t])
+      af[t] = AT ? load_frag_f32<ADD>(Af + aoff[t] + k, a_add + aoff[t] + k, ok && a_live[t], ss[t])
                  : load_frag(Ab + aoff[t] + k, ok && a_live[t]);
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -357,7 +391,10 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       }
       EpiOperands fresh;
       fresh.have = false;
-      store_tile<EPI>(s, m, n, N, ldc, Cv, rp, PRE ? pre[j] : fresh);
+      if (EPI == 2 && second)
+        store_tile<0>(s, m, n, N, ldc, rd.half_out, nullptr, rp, fresh);
+      else
+        store_tile<EPI>(s, m, n, N, ldc, Cv, c_add, rp, PRE ? pre[j] : fresh);
     }
   }
 }
@@ -378,14 +415,24 @@ int pick_waves(int K) {
 
 template <int MT, int NT, int AT, int EPI>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-               int m_base, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
+               int m_base, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   int nw = pick_waves(K);
   if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
-  const dim3 grid(groups), block(nw * KVF_WAVE);
+  const dim3 grid(groups, EPI == 2 && rd.half_out ? 2 : 1), block(nw * KVF_WAVE);
   const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI>), grid, block, lds, s, A, W, C, M, N, K,
-                     lda, ldc, m_base, eps, w_tiled, rp);
+  if (rd.a_add) {
+    // the sum that rides in the left operand's loads: only the fused q/k/v projection of one
+    // tile of rows is built with it
+    if constexpr (MT == 1 && AT == 1 && EPI == 4)
+      hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, true>), grid, block, lds, s, A, W, C, M, N, K,
+                         lda, ldc, m_base, eps, w_tiled, rd, rp);
+    else
+      return static_cast<int>(hipErrorInvalidValue);
+  } else {
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, false>), grid, block, lds, s, A, W, C, M, N, K,
+                       lda, ldc, m_base, eps, w_tiled, rd, rp);
+  }
   return kvf_last_error();
 }
 
@@ -393,47 +440,47 @@ int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int
 // spare (the grid must still fill the chip).
 template <int MT, int AT, int EPI>
 int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-              int m_base, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
+              int m_base, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
   const int tiles = (N + 15) / 16;
   if (MT >= 2 && MT <= 4 && !AT) {
     if (MT == 4 && tiles >= 1024)
-      return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+      return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
     if (tiles >= 512)
-      return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+      return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
   }
   if (MT == 1) {
     // Every workgroup reads all of A, so with several rows of A and many rows of W a workgroup
     // takes 32 rows of W and halves that traffic.
     const int rw = g_rows_override > 0 ? g_rows_override : (M - m_base > 4 && tiles >= 512 ? 32 : 16);
-    if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
-    if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
+    if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
   }
-  return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+  return launch_one<MT, 1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
 }
 
 template <int AT, int EPI>
 int launch_rows(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-                float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
+                float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
   int err = 0;
   for (int m_base = 0; m_base < M && !err; m_base += 128) {
     const int rows = M - m_base < 128 ? M - m_base : 128;
-    if (rows <= 16) err = launch_nt<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
-    else if (rows <= 32) err = launch_nt<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
-    else if (rows <= 64) err = launch_nt<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
-    else err = launch_nt<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rp, s);
+    if (rows <= 16) err = launch_nt<1, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
+    else if (rows <= 32) err = launch_nt<2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
+    else if (rows <= 64) err = launch_nt<4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
+    else err = launch_nt<8, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
   }
   return err;
 }
 
 template <int AT>
 int launch_epi(const void* A, const bf16_t* W, void* C, int epi, int M, int N, int K, int lda,
-               int ldc, float eps, int w_tiled, const RopeEpi& rp, hipStream_t s) {
+               int ldc, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
   switch (epi) {
-    case 0: return launch_rows<AT, 0>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
-    case 1: return launch_rows<AT, 1>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
-    case 2: return launch_rows<AT, 2>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
-    case 3: return launch_rows<AT, 3>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
-    case 4: return launch_rows<AT, 4>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rp, s);
+    case 0: return launch_rows<AT, 0>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+    case 1: return launch_rows<AT, 1>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+    case 2: return launch_rows<AT, 2>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+    case 3: return launch_rows<AT, 3>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+    case 4: return launch_rows<AT, 4>(A, W, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
   }
   return static_cast<int>(hipErrorInvalidValue);
 }
@@ -447,37 +494,48 @@ KVF_EXPORT void kvf_gemm_bf16_set_rows(int rows) { g_rows_override = rows; }
 // a_type: 0 = bf16 rows, 1 = fp32 rows normalised by rsqrt(mean(x^2) + eps) in the kernel.
 // epi: 0 store fp32, 1 store bf16, 2 add into fp32, 3 SwiGLU pairs -> bf16 [M, N/2].
 // w_tiled: W is [N, K] row-major (0) or in tiles of 16 x 32 (1, see the head of this file).
+// c_add (epi 2 only, may be null): fp32 [M, ldc], added to C together with the product.
+// half_out (epi 2 with bf16 rows only, may be null): fp32 [M, ldc]; the product over the second
+//   half of K is stored there instead of being added to C, by a second layer of workgroups.
 KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, int w_tiled, void* C, int epi,
-                             int M, int N, int K, int lda, int ldc, float eps, hipStream_t s) {
+                             int M, int N, int K, int lda, int ldc, float eps, const float* c_add,
+                             float* half_out, hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || epi < 0 || epi > 3 || (epi == 3 && N % 4 != 0))
     return static_cast<int>(hipErrorInvalidValue);
+  if (((c_add || half_out) && epi != 2) || (half_out && (a_type != 0 || K < 64)))
+    return static_cast<int>(hipErrorInvalidValue);
   const RopeEpi none{};
+  const Riders rd{nullptr, c_add, half_out};
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, none, s);
-  if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, none, s);
+  if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, rd, none, s);
+  if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, rd, none, s);
   return static_cast<int>(hipErrorInvalidValue);
 }
 
 // Fused q/k/v projection with rotary and cache write.  W: [(H + 2*KV) * d, K] with q and k rows
 // permuted so that rotary pairs are neighbouring rows.  q_out: [M, ldq >= H * d] bf16.
+// a_add (a_type 1 and at most 16 rows only, may be null): fp32 [M, lda], added to A before the
+// norm.
 KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, int w_tiled,
                                       void* q_out, int M, int K, int lda, int ldq, float eps,
-                                      const int* positions,
+                                      const float* a_add, const int* positions,
                                       const int* seq_of_token, const float* cos_t,
                                       const float* sin_t, const int* block_table, void* k_pages,
                                       void* v_pages, int H, int KV, int d, int rot, int table_len,
                                       int block_size, int table_stride, int num_blocks,
                                       int write_kv, int n_seqs, hipStream_t s) {
   if (M <= 0) return 0;
-  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || d % 4 != 0 || rot % 2 != 0 || rot > d || ldq % 4 != 0)
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || d % 4 != 0 || rot % 2 != 0 || rot > d || ldq % 4 != 0 ||
+      (a_add && (a_type != 1 || M > 16)))
     return static_cast<int>(hipErrorInvalidValue);
+  const Riders rd{a_add, nullptr, nullptr};
   const RopeEpi rp{positions, seq_of_token, cos_t, sin_t, block_table,
                    static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), H, KV, d, rot,
                    table_len, block_size, table_stride, num_blocks, write_kv, n_seqs};
   const int N = (H + 2 * KV) * d;
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rp, s);
-  if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rp, s);
+  if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);
+  if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);
   return static_cast<int>(hipErrorInvalidValue);
 }

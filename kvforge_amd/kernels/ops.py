@@ -91,8 +91,8 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch
             rows: torch.Tensor | None = None, add: torch.Tensor | None = None) -> None:
     """``out[m] = y * rsqrt(mean(y^2) + eps) * weight`` with ``y = x[rows[m] or m]`` in fp32
     (``weight=None``: no weight, for a norm whose weight is folded into the next matrix).
-    ``add`` (``[rows of x, h]``, dtype of ``out``) is a sum still owed to ``x``: the norm is taken
-    of ``x + add``, and without ``rows`` the sum is written back to ``x`` as well."""
+    ``add`` (``[rows of x, h]``, dtype of ``out`` or fp32) is a sum still owed to ``x``: the norm
+    is taken of ``x + add``, and without ``rows`` the sum is written back to ``x`` as well."""
     _check(x, "x", F32, (None, None))
     xr, h = x.shape
     m = out.shape[0]
@@ -106,12 +106,15 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch
     elif m > xr:
         raise KernelError("rmsnorm: more output rows than input rows")
     if add is not None:
-        _check(add, "add", out.dtype, (xr, h))
+        _check(add, "add", None, (xr, h))
+        if add.dtype not in (F32, out.dtype):
+            raise KernelError(f"rmsnorm: add must be float32 or {out.dtype}, got {add.dtype}")
     f = _fn("elementwise", f"kvf_rmsnorm_{_suffix(out.dtype)}",
-            [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int,
-             c_void_p])
+            [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_float, c_void_p, c_int, c_int,
+             c_int, c_void_p])
     _ok(f(x.data_ptr(), rows.data_ptr() if rows is not None else None,
           add.data_ptr() if add is not None else None,
+          1 if add is not None and add.dtype == F32 else 0,
           weight.data_ptr() if weight is not None else None,
           1 if weight is not None and weight.dtype == F32 else 0, float(eps), out.data_ptr(),
           m, h, xr, _stream()), "rmsnorm")
@@ -184,7 +187,13 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
 SKINNY_MAX_M = 32
 FUSED_NORM_MAX_M = 16
 FUSED_EPILOGUE_MAX_M = 64
-_GEMM_BF16_ARGS = [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_float, c_void_p]
+_GEMM_BF16_ARGS = ([c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6
+                   + [c_float, c_void_p, c_void_p, c_void_p])
+# A product that is added to a narrow fp32 stream (few output columns, long K) has too few
+# workgroups to pull on the weights with all of the chip: below this many groups of 16 columns
+# and from this K on it is cut into two halves of K (``k_halves_pay``).
+K_HALVES_MAX_GROUPS = 192
+K_HALVES_MIN_K = 4096
 
 
 class StreamedWeight:
@@ -281,16 +290,40 @@ def is_library_product(a: torch.Tensor, w: torch.Tensor) -> bool:
             and (m > SKINNY_MAX_M or (m > 16 and k >= 2 * n)))
 
 
-def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> None:
+def k_halves_pay(a: torch.Tensor, w) -> bool:
+    """Whether ``gemm(a, w, out, accumulate=True, half_out=...)`` is worth asking for: one tile of
+    bf16 rows over a deep weight with few columns (the down projection of a small model)."""
+    m, k = a.shape
+    return (not is_library_product(a, w) and a.dtype == BF16 and plain_of(w).dtype == BF16
+            and k % 8 == 0 and m <= 16 and k >= K_HALVES_MIN_K
+            and -(-w.shape[0] // 16) <= K_HALVES_MAX_GROUPS)
+
+
+def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
+         owed: torch.Tensor | None = None, half_out: torch.Tensor | None = None) -> None:
     """``out = a @ w.T`` (``accumulate``: ``out += a @ w.T`` with ``out`` fp32).
 
     ``a: [M, K]`` (row stride may exceed K), ``w: [N, K]`` contiguous or a ``StreamedWeight``,
     ``out: [M, N]``.
     bf16 x bf16 runs on MFMA with fp32 accumulation; any operand in fp32 runs the fp32
-    vector-ALU kernel (true 32-bit multiply and accumulate)."""
+    vector-ALU kernel (true 32-bit multiply and accumulate).
+    With ``accumulate``: ``owed`` (fp32, like ``out``) is a sum still owed to ``out`` and is added
+    on the way; ``half_out`` (fp32, like ``out``, only where ``k_halves_pay``) receives the
+    product over the second half of K *instead of* ``out``, which the caller then owes to
+    ``out``: twice the workgroups pull on ``w``."""
     m, n, k, lda, ldc = _gemm_operands(a, w, out, lambda n: n)
     if accumulate and out.dtype != F32:
         raise KernelError("gemm: accumulation needs an fp32 output")
+    for t, name in ((owed, "owed"), (half_out, "half_out")):
+        if t is None:
+            continue
+        if not accumulate:
+            raise KernelError(f"gemm: {name} goes with accumulate")
+        _check(t, name, F32, (m, n), contiguous=False)
+        if t.stride(1) != 1 or (m > 1 and t.stride(0) != ldc):
+            raise KernelError(f"gemm: {name} must have the row stride of out")
+    if half_out is not None and not k_halves_pay(a, w):
+        raise KernelError("gemm: half_out only where k_halves_pay(a, w)")
     if m == 0:
         return
     out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)
@@ -301,8 +334,12 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> Non
             f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
             wp, tiled = _w_args(w)
             _ok(f(a.data_ptr(), 0, wp, tiled, out.data_ptr(), out_kind, m, n, k, lda, ldc, 0.0,
-                  _stream()), "gemm_bf16")
-        elif accumulate:
+                  owed.data_ptr() if owed is not None else None,
+                  half_out.data_ptr() if half_out is not None else None, _stream()), "gemm_bf16")
+            return
+        if owed is not None:
+            out.add_(owed)
+        if accumulate:
             # many rows: the library's bf16 product, then the residual sum in fp32
             out.add_(torch.mm(a, plain_of(w).t()))
         elif out.dtype == F32:
@@ -310,6 +347,8 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False) -> Non
         else:
             torch.mm(a, plain_of(w).t(), out=out)
         return
+    if owed is not None:
+        out.add_(owed)
     w = plain_of(w)
     f = _fn("gemm_generic", "kvf_gemm_generic",
             [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_void_p])
@@ -345,17 +384,19 @@ def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: flo
     f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
     wp, tiled = _w_args(w)
     _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, out.data_ptr(), epi, m, n, k, lda, ldc,
-          float(rms_eps or 0.0), _stream()), "gemm_bf16")
+          float(rms_eps or 0.0), None, None, _stream()), "gemm_bf16")
 
 
 def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
                   seq_of_token: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                   block_table: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True,
-                  rms_eps: float | None = None) -> None:
+                  rms_eps: float | None = None, a_owed: torch.Tensor | None = None) -> None:
     """Fused q/k/v projection: ``a @ w.T`` with rotary applied to q and k (neighbouring columns
     are pairs), rotated q stored to ``q_out [M, H*d]`` and rotated k and v written into the
-    pages.  ``rms_eps`` as in ``gemm_fused``."""
+    pages.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; fp32, shape and
+    strides of ``a``): a sum still owed to ``a``; the projection is taken of ``a + a_owed``, and
+    ``a`` itself is left as it is."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     rms = rms_eps is not None
     m, k = a.shape
@@ -363,6 +404,12 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     _check(plain_of(w), "w", BF16, ((H + 2 * KV) * d, k))
     if not bf16_kernel_takes(a, w, rms, True) or a.stride(1) != 1:
         raise KernelError("gemm_qkv_rope: operands do not fit the MFMA kernel")
+    if a_owed is not None:
+        if not rms or m > FUSED_NORM_MAX_M:
+            raise KernelError("gemm_qkv_rope: a_owed goes with rms_eps (fp32 rows, one tile of them)")
+        _check(a_owed, "a_owed", F32, (m, k), contiguous=False)
+        if a_owed.stride() != a.stride():
+            raise KernelError("gemm_qkv_rope: a_owed must have the strides of a")
     _check(q_out, "q_out", BF16, (m, H * d))
     _check(positions, "positions", I32, (None,))
     _check(seq_of_token, "seq_of_token", I32, (None,))
@@ -381,11 +428,11 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
         return
     f = _fn("gemm_bf16", "kvf_gemm_bf16_qkv_rope",
             [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float]
-            + [c_void_p] * 7 + [c_int] * 10 + [c_void_p])
+            + [c_void_p] * 8 + [c_int] * 10 + [c_void_p])
     wp, tiled = _w_args(w)
     _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, q_out.data_ptr(), m, k,
           a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d, float(rms_eps or 0.0),
-          positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+          a_owed.data_ptr() if a_owed is not None else None, positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(), sin.data_ptr(),
           block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, 2 * half,
           table_len, bs, block_table.shape[1], nb, 1 if write_kv else 0, block_table.shape[0],
           _stream()), "gemm_qkv_rope")

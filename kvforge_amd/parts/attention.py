@@ -105,20 +105,30 @@ class PagedAttention(Mixer):
         table = step.block_tables[layer.group]
         cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else step.no_rotation()
         rms = self.norm_eps
+        owed = None
         if rms is not None and not ops.bf16_kernel_takes(x, self.w_qkv, True):
             # too many rows for the norm to ride in the projection: a norm kernel of its own,
             # which also adds what the layer before still owes the stream
             normed = ws.buf("normed", (n, self.hidden), act)
             ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
+        fused = (ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
+                 and layer.k_pages.dtype == torch.bfloat16)
+        if fused and rms is not None:
+            # what the layer before owes the stream in fp32 rides in this projection's loads and
+            # is added to the stream by the output projection
+            owed = step.take_owed(residual)
+            if owed is not None and owed.dtype != torch.float32:
+                ops.add_rows(residual, owed)
+                owed = None
         else:
             step.settle()
-        if ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True) and layer.k_pages.dtype == torch.bfloat16:
+        if fused:
             # one kernel: (norm,) projection, rotary, cache write
             qkv = ws.buf("q_rot", (n, H * d), act)
             ops.gemm_qkv_rope(x, self.w_qkv, qkv, step.positions, step.seq_of_token, cos, sin, table,
                               layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache,
-                              rms_eps=rms)
+                              rms_eps=rms, a_owed=owed)
         else:
             qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), act)
             ops.gemm(x, self.w_qkv, qkv)
@@ -137,4 +147,4 @@ class PagedAttention(Mixer):
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None)
-        add_product(step, out, self.w_o, residual)
+        add_product(step, out, self.w_o, residual, owed=owed)

@@ -187,19 +187,30 @@ class Block(Part):
         return all(p.replayable for p in self.parts())
 
 
-def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor) -> None:
+def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor,
+                owed: torch.Tensor | None = None) -> None:
     """``residual += a @ w.T``, the last product of a mixer or feed-forward.  With few rows (or in
     fp32) the product kernel adds in its epilogue.  Many bf16 rows go to the library, whose
     product is left owed to the stream (``step.owe``) so that the next norm adds it on its way
-    instead of an add kernel of its own."""
+    instead of an add kernel of its own.  One tile of rows over a deep weight with few columns
+    is cut into two halves of K so that every compute unit pulls on the weight: the first half
+    is added here, the second is left owed (in fp32).
+    ``owed``: a sum the caller took from the step (``step.take_owed``) and has not added yet;
+    it is added here, in the same kernel where that is possible."""
     from kvforge_amd.kernels import ops
 
     if ops.is_library_product(a, w):
+        if owed is not None:
+            ops.add_rows(residual, owed)
         product = step.ws.buf("owed_product", (a.shape[0], w.shape[0]), a.dtype)
         ops.gemm(a, w, product)
         step.owe(residual, product)
+    elif ops.k_halves_pay(a, w) and residual.is_contiguous():
+        half = step.ws.buf("owed_half", tuple(residual.shape), torch.float32)
+        ops.gemm(a, w, residual, accumulate=True, owed=owed, half_out=half)
+        step.owe(residual, half)
     else:
-        ops.gemm(a, w, residual, accumulate=True)
+        ops.gemm(a, w, residual, accumulate=True, owed=owed)
 
 
 @dataclass(frozen=True)

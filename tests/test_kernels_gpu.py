@@ -42,11 +42,13 @@ def test_embed(dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("h", [96, 100, 2048, 5000])
-def test_rmsnorm_with_owed_sum(dtype, h):
-    """norm(x + add): without rows the sum is left in x; with rows x stays as it was."""
+@pytest.mark.parametrize("add32", [False, True])
+def test_rmsnorm_with_owed_sum(dtype, h, add32):
+    """norm(x + add): without rows the sum is left in x; with rows x stays as it was.  The sum
+    owed is in the output's type (a library product) or in fp32 (half of a product cut in K)."""
     g = torch.Generator().manual_seed(h + 1)
     x = torch.randn(7, h, generator=g) * 2
-    add = torch.randn(7, h, generator=g).to(dtype)
+    add = torch.randn(7, h, generator=g).to(torch.float32 if add32 else dtype)
     w = (1 + 0.1 * torch.randn(h, generator=g)).to(dtype)
     total = x + add.float()
     xd = x.to(DEV)
@@ -204,6 +206,43 @@ def test_gemm_over_tiled_weights_gives_the_same_bits(m, n, k):
     assert torch.equal(o1, o2)
 
 
+@pytest.mark.parametrize("m", [1, 7, 16])
+@pytest.mark.parametrize("n,k", [(2048, 8192), (100, 4096), (3072, 4104)])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_gemm_cut_in_two_halves_of_k(m, n, k, tiled):
+    """out += a @ w.T with the second half of K left in half_out, and a sum owed to out added on
+    the way: out + half_out is the whole sum; every value is an fp32 sum in a fixed order, so a
+    second call gives the same bits."""
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16).to(DEV)
+    w = ops().StreamedWeight(w) if tiled else w
+    res = torch.randn(m, n, generator=g)
+    owed = torch.randn(m, n, generator=g)
+    assert ops().k_halves_pay(a.to(DEV), w)
+    cut = (-(-k // 32) + 1) // 2 * 32                    # the first half takes the odd k-step
+    first = a[:, :cut].double() @ ops().plain_of(w).cpu()[:, :cut].double().T
+    second = a[:, cut:].double() @ ops().plain_of(w).cpu()[:, cut:].double().T
+    outs = []
+    for _ in range(2):
+        out, half = res.clone().to(DEV), torch.full((m, n), 7.0, device=DEV)
+        ops().gemm(a.to(DEV), w, out, accumulate=True, owed=owed.to(DEV), half_out=half)
+        torch.testing.assert_close(out.double().cpu(), res.double() + owed.double() + first, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(half.double().cpu(), second, atol=1e-4, rtol=1e-4)
+        outs.append((out, half))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # the sum owed alone, without the cut
+    out = res.clone().to(DEV)
+    ops().gemm(a.to(DEV), w, out, accumulate=True, owed=owed.to(DEV))
+    torch.testing.assert_close(out.double().cpu(), res.double() + owed.double() + first + second,
+                               atol=1e-4, rtol=1e-4)
+    with pytest.raises(ops().KernelError):
+        ops().gemm(a.to(DEV), w, torch.empty(m, n, device=DEV), half_out=torch.empty(m, n, device=DEV))
+    with pytest.raises(ops().KernelError):               # a shallow weight is not cut
+        ops().gemm(a.to(DEV)[:, :64].contiguous(), ops().plain_of(w)[:, :64].contiguous(), res.clone().to(DEV),
+                   accumulate=True, half_out=torch.empty(m, n, device=DEV))
+
+
 @pytest.mark.parametrize("m", [1, 8, 16, 20, 33, 50, 64])
 @pytest.mark.parametrize("n,k", [(352, 96), (512, 2048), (48, 40)])
 def test_gemm_fused_norm_and_gate(m, n, k):
@@ -307,6 +346,18 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     assert once.any()
     untouched = (kp_ref.float().cpu().abs().sum((1, 3)) == 0)
     assert (kp.float().cpu().abs().sum((1, 3))[untouched] == 0).all()
+    if rms:
+        # a sum still owed to the rows rides in the loads: the same bits as rows summed before,
+        # and the rows themselves stay as they were
+        a1, a2 = torch.randn(m, k, generator=g), torch.randn(m, k, generator=g)
+        got = []
+        for rows, owed in (((a1 + a2).to(DEV), None), (a1.to(DEV), a2.to(DEV))):
+            kp2, vp2, q2 = torch.zeros_like(kp_ref), torch.zeros_like(vp_ref), torch.empty_like(q)
+            ops().gemm_qkv_rope(rows, w, q2, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV),
+                                kp2, vp2, H, KV, d, rms_eps=eps, a_owed=owed)
+            got.append((q2, kp2.cpu()[sel], vp2.cpu()[sel_v]))
+            assert torch.equal(rows.cpu(), a1 if owed is not None else a1 + a2)
+        assert all(torch.equal(x1, x2) for x1, x2 in zip(*got))
 
 
 def test_gemm_bf16_rows_do_not_depend_on_neighbours():
