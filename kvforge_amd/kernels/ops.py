@@ -190,9 +190,11 @@ FUSED_EPILOGUE_MAX_M = 64
 _GEMM_BF16_ARGS = ([c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6
                    + [c_float, c_void_p, c_void_p, c_void_p])
 # A product that is added to a narrow fp32 stream (few output columns, long K) has too few
-# workgroups to pull on the weights with all of the chip: below this many groups of 16 columns
-# and from this K on it is cut into two halves of K (``k_halves_pay``).
-K_HALVES_MAX_GROUPS = 192
+# workgroups to pull on the weights with all of the chip: with at most this many groups of 16
+# columns (half the compute units) and from this K on it is cut into two halves of K
+# (``k_halves_pay``).  The half that is left owed costs its consumers a second fp32 operand, so
+# wider streams lose more there than the product gains (measured at 3072 columns: 7% of the step).
+K_HALVES_MAX_GROUPS = 128
 K_HALVES_MIN_K = 4096
 
 
