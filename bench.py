@@ -76,15 +76,19 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
     while any(r.is_prefill for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
         engine.step()
     run_limit = engine.config.decode_run_steps
+    run_ahead = engine.config.decode_run_ahead
 
     def decode_steps(n):
         """Exactly ``n`` decode steps of the whole batch (the engine may take several between two
-        looks of the host; the last run is cut to fit); returns the tokens produced."""
+        looks of the host; the last run is cut to fit, and no run is queued ahead that these
+        ``n`` steps would not read); returns the tokens produced."""
         produced, start = 0, engine.runner.num_forward_passes
         while engine.runner.num_forward_passes - start < n:
-            engine.config.decode_run_steps = min(run_limit, n - (engine.runner.num_forward_passes - start))
+            left = n - (engine.runner.num_forward_passes - start)
+            engine.config.decode_run_steps = min(run_limit, left)
+            engine.config.decode_run_ahead = run_ahead and left >= 2 * run_limit
             produced += sum(len(o.new_token_ids) for o in engine.step())
-        engine.config.decode_run_steps = run_limit
+        engine.config.decode_run_steps, engine.config.decode_run_ahead = run_limit, run_ahead
         assert engine.runner.num_forward_passes - start == n
         return produced
 
@@ -173,7 +177,7 @@ def main() -> int:
         batches = [args.batch] + ([b for b in (1, 64) if b != args.batch] if points else [])
         prefill_s = None
         for b in batches:
-            need = b * (args.prompt_len + args.steps + args.warmup + early_tokens(b, args.prompt_len) + 16)
+            need = b * (args.prompt_len + args.steps + args.warmup + early_tokens(b, args.prompt_len) + 32)
             engine = build_engine(folder, args.dtype, max(b, 1), max(need, PREFILL_TOKENS + 64),
                                   use_graphs=not args.no_graphs, run_steps=args.decode_run_steps,
                                   context_cap=args.context_len)

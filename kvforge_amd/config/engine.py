@@ -75,6 +75,11 @@ class EngineConfig:
     # steps by itself (each sampled token becomes the next input there) before the host reads
     # the tokens and looks at stop conditions; 1 makes the host look after every step.
     decode_run_steps: int = 8
+    # While such runs follow each other for the same requests, queue the next run on the device
+    # before the tokens of the current one are read, so that the device does not wait for the
+    # host in between.  A run that turns out not to be wanted (a request stopped, another one
+    # arrived) is left unread; what it wrote to the cache is computed again by the next step.
+    decode_run_ahead: bool = True
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)

@@ -229,6 +229,66 @@ class Step:
         return splits, (acc, ml)
 
 
+def _fill_tables(meta: "MetaBuffers", host: np.ndarray, entries: Sequence[StepEntry], Bp: int,
+                 need_tokens: Sequence[int], tables_of, block_size: int,
+                 windowed_groups: Sequence[bool] | None, serial_of) -> int:
+    """Bring the host mirror of the block tables up to date for ``entries`` (row ``b`` holds the
+    pages of ``need_tokens[b]`` positions; rows ``len(entries)..Bp-1`` are empty) and write the
+    rows into the staging memory ``host``.  Returns the end of the table region."""
+    B = len(entries)
+    end = 0
+    for g, (to, w) in enumerate(zip(meta.table_off, meta.table_widths)):
+        mirror, owner, filled = meta.table_host[g], meta.row_owner[g], meta.row_filled[g]
+        windowed = windowed_groups is not None and windowed_groups[g]
+        for b, e in enumerate(entries):
+            t = tables_of(e.request_id, g)
+            need = -(-need_tokens[b] // block_size)
+            if need > w or need > len(t):
+                raise ValueError(f"request {e.request_id} needs {need} pages in group {g}; "
+                                 f"table holds {len(t)}, width {w}")
+            have = int(filled[b])
+            tag = (e.request_id, serial_of(e.request_id)) if serial_of is not None else None
+            if tag is not None and owner[b] == tag and have <= need and not windowed:
+                if have < need:
+                    mirror[b, have:need] = t[have:need]
+            else:
+                mirror[b, :have] = -1
+                mirror[b, :need] = t[:need]
+                owner[b] = tag
+            filled[b] = need
+        for b in range(B, Bp):
+            if filled[b]:
+                mirror[b, :int(filled[b])] = -1
+            owner[b], filled[b] = None, 0
+        host[to:to + Bp * w].reshape(Bp, w)[:] = mirror[:Bp]
+        end = to + Bp * w
+    return end
+
+
+def extend_tables(meta: "MetaBuffers", entries: Sequence[StepEntry], padded: int,
+                  need_tokens: Sequence[int], tables_of, block_size: int,
+                  windowed_groups: Sequence[bool] | None = None, serial_of=None) -> None:
+    """For a batch that is on the device already (same entries, same rows): make its block
+    tables hold the pages of ``need_tokens[b]`` positions.  Only the table region travels, in
+    stream order, so launches queued before it still see the tables they were queued with (it
+    only adds pages, or takes away pages that lie wholly behind a window)."""
+    if not meta.table_off:
+        return
+    turn = meta.turn
+    meta.turn ^= 1
+    if meta.events[turn] is not None:
+        meta.events[turn].synchronize()
+    host = meta.staging_np[turn]
+    end = _fill_tables(meta, host, entries, padded, need_tokens, tables_of, block_size,
+                       windowed_groups, serial_of)
+    start = meta.table_off[0]
+    meta.device_buf[start:end].copy_(meta.staging[turn][start:end], non_blocking=True)
+    if meta.device_buf.is_cuda:
+        ev = meta.events[turn] or torch.cuda.Event()
+        ev.record()
+        meta.events[turn] = ev
+
+
 def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], tables_of, slot_of,
               block_size: int, pad_to: int | None = None,
               windowed_groups: Sequence[bool] | None = None, serial_of=None,
@@ -297,31 +357,9 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
     host[off["decode_seq_ids"]:off["decode_seq_ids"] + len(decode)] = decode
 
     end = off["logits_rows"] + max(R, 1)
-    for g, (to, w) in enumerate(zip(meta.table_off, meta.table_widths)):
-        mirror, owner, filled = meta.table_host[g], meta.row_owner[g], meta.row_filled[g]
-        windowed = windowed_groups is not None and windowed_groups[g]
-        for b, e in enumerate(entries):
-            t = tables_of(e.request_id, g)
-            need = -(-(int(ctx[b]) + lookahead) // block_size)
-            if need > w or need > len(t):
-                raise ValueError(f"request {e.request_id} needs {need} pages in group {g}; "
-                                 f"table holds {len(t)}, width {w}")
-            have = int(filled[b])
-            tag = (e.request_id, serial_of(e.request_id)) if serial_of is not None else None
-            if tag is not None and owner[b] == tag and have <= need and not windowed:
-                if have < need:
-                    mirror[b, have:need] = t[have:need]
-            else:
-                mirror[b, :have] = -1
-                mirror[b, :need] = t[:need]
-                owner[b] = tag
-            filled[b] = need
-        for b in range(B, Bp):
-            if filled[b]:
-                mirror[b, :int(filled[b])] = -1
-            owner[b], filled[b] = None, 0
-        host[to:to + Bp * w].reshape(Bp, w)[:] = mirror[:Bp]
-        end = to + Bp * w
+    need_tokens = [int(ctx[b]) + lookahead for b in range(B)]
+    end = max(end, _fill_tables(meta, host, entries, Bp, need_tokens, tables_of, block_size,
+                                windowed_groups, serial_of))
     meta.device_buf[:end].copy_(meta.staging[turn][:end], non_blocking=True)
     if meta.device_buf.is_cuda:
         ev = meta.events[turn] or torch.cuda.Event()

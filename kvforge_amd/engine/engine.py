@@ -125,42 +125,51 @@ class InferenceEngine:
         sched = self.scheduler.schedule()
         if sched.is_empty:
             return []
-        run = self._decode_run_length(sched)
-        new_tokens = self._run(sched.scheduled, run)
+        run, ahead = self._decode_run_length(sched)
+        new_tokens = self._run(sched.scheduled, run, ahead)
         outputs = self._postprocess(sched.scheduled, new_tokens)
         self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens * run,
                                  time.perf_counter() - t0,
                                  1.0 - self.cache.num_free_blocks / max(1, self.cache.num_blocks))
         return outputs
 
-    def _decode_run_length(self, sched) -> int:
+    def _decode_run_length(self, sched) -> tuple[int, bool]:
         """How many decode steps the device takes before the host looks again: more than one
         only while every scheduled request decodes, nobody waits for admission, no request can
-        reach its length limit inside the run, and the pages of the run's positions are free."""
+        reach its length limit inside the run, and the pages of the run's positions are free.
+        The second value says that all of this also holds for the run after it, whose pages are
+        then allocated as well, so that the runner may queue that run before this one is read
+        (``EngineConfig.decode_run_ahead``)."""
         limit = self.config.decode_run_steps
         group = sched.scheduled
         if (limit <= 1 or sched.preempted or self.scheduler.num_waiting
                 or any(s.is_prefill or s.num_new_tokens != 1 for s in group)):
-            return 1
+            return 1, False
         max_len = self.config.scheduler.max_model_len
-        for s in group:
-            r = s.request
-            limit = min(limit, r.sampling_params.max_tokens - r.num_output_tokens,
-                        max_len - r.num_tokens)
+        room = min(min(s.request.sampling_params.max_tokens - s.request.num_output_tokens,
+                       max_len - s.request.num_tokens) for s in group)
+        limit = min(limit, room)
         if limit <= 1:
-            return 1
+            return 1, False
         entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
                    for s in group]
         if not self.runner.graph_takes(entries, len(entries)):
-            return 1
+            return 1, False
         wanted = [(s.request.request_id, s.request.num_computed_tokens + limit) for s in group]
         if not self.cache.can_append_all(wanted):
-            return 1
+            return 1, False
+        ahead = self.config.decode_run_ahead and limit == self.config.decode_run_steps and room >= 2 * limit
+        if ahead:
+            further = [(rid, total + limit) for rid, total in wanted]
+            ahead = self.cache.can_append_all(further)
+            if ahead:
+                wanted = further
         for s, (rid, total) in zip(group, wanted):
             self.cache.append_slots(rid, total, s.request.num_computed_tokens)
-        return limit
+        return limit, ahead
 
-    def _run(self, group: list[ScheduledRequest], run: int = 1) -> dict[str, list[int]]:
+    def _run(self, group: list[ScheduledRequest], run: int = 1, ahead: bool = False
+             ) -> dict[str, list[int]]:
         if run > 1:
             reqs = [s.request for s in group]
             entries = [StepEntry(r.request_id, r.token_slice(r.num_computed_tokens, 1),
@@ -168,7 +177,7 @@ class InferenceEngine:
             steps = self.runner.decode_run(entries, self.sampler.seed,
                                            [r.sampling_params for r in reqs],
                                            [r.sample_stream for r in reqs],
-                                           [r.num_output_tokens for r in reqs], run)
+                                           [r.num_output_tokens for r in reqs], run, ahead)
             for r in reqs:
                 r.num_computed_tokens += 1
             return {r.request_id: [step[i] for step in steps] for i, r in enumerate(reqs)}

@@ -16,8 +16,9 @@ import torch
 
 from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
-from kvforge_amd.engine.batch import (DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS, MetaBuffers, Step, StepEntry,
-                                      Workspace, fill_step)
+from kvforge_amd.engine.batch import (DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS, MetaBuffers, Step,
+                                      StepEntry, Workspace, fill_step,
+                                      extend_tables)
 from kvforge_amd.kernels import ops
 from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
@@ -68,6 +69,11 @@ class ModelRunner:
         # tickets and chunk results of greedy rows read by several workgroups (zero between launches)
         self._sample_work = torch.zeros(ops.sample_work_size(cap), dtype=torch.int32, device=self.device)
         self._run_ring = torch.zeros(MAX_DECODE_RUN, cap, dtype=torch.int32, device=self.device)
+        self._ring_host = torch.zeros(MAX_DECODE_RUN, cap, dtype=torch.int32, pin_memory=True)
+        self._ring_host_np = self._ring_host.numpy()
+        self._queued: _QueuedRun | None = None   # a run queued ahead of the call that will read it
+        self.num_runs_queued_ahead = 0
+        self.num_runs_read_ahead = 0
         self._sample_f_host = torch.zeros(nf, dtype=torch.float32, pin_memory=True)
         self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
         self._sample_f_np, self._sample_i_np = self._sample_f_host.numpy(), self._sample_i_host.numpy()
@@ -98,6 +104,7 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """One forward over the entries; fp32 logits ``[sum of wanted places, vocab]``, rows in
         entry order then place order.  The tensor is a view of memory the next step reuses."""
+        self._queued = None  # whatever is queued ahead is not what comes next
         step, _ = self.build_step(entries)
         logits = self.model.forward(step)
         self.num_forward_passes += 1
@@ -124,8 +131,8 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ decode through graphs
     @torch.inference_mode()
-    def decode_run(self, entries, seed, params, streams, counters, num_steps: int = 1
-                   ) -> list[list[int]]:
+    def decode_run(self, entries, seed, params, streams, counters, num_steps: int = 1,
+                   ahead: bool = False) -> list[list[int]]:
         """``num_steps`` decode steps of single tokens with one wait for the device at the end;
         returns the tokens of every step, ``[step][entry]``.
 
@@ -133,18 +140,49 @@ class ModelRunner:
         graph and replayed: metadata and sampling parameters live at fixed device addresses and
         are refreshed by two copies before the run.  The graph ends with a kernel that turns each
         sampled token into the sequence's next input, so further steps need nothing from the
-        host; the pages of their positions must be in the requests' tables already."""
+        host; the pages of their positions must be in the requests' tables already.
+
+        ``ahead``: the caller expects to come back for the same requests, ``num_steps`` further
+        on, with the pages of those positions allocated already (twice ``num_steps`` from here).
+        The runner then queues that next run before it waits for this one, so the device goes on
+        while the host looks at the tokens; a next call that is this continuation finds its run
+        queued.  Any other call simply leaves the queued run to finish unread: its launches only
+        rewrite cache positions that the next real step computes again, in stream order before
+        it.  (Not for models with per-request state, which a discarded run would advance.)"""
         b = len(entries)
         k = int(num_steps)
         if not 1 <= k <= MAX_DECODE_RUN:
             raise ValueError(f"a run holds 1 to {MAX_DECODE_RUN} steps")
         if not self.graph_takes(entries, len(params)):
             raise ValueError("a decode run takes single tokens that each want their logits")
+        queued, self._queued = self._queued, None
+        ids = [e.request_id for e in entries]
+        if (queued is not None and queued.ids == ids and queued.k == k
+                and queued.begins == [e.start_pos for e in entries]):
+            run = queued
+            self.num_runs_read_ahead += 1
+        else:
+            run = self._launch_run(entries, seed, params, streams, counters, k,
+                                   lookahead=(2 * k if ahead else k) - 1)
+        if ahead and 2 * k <= MAX_DECODE_RUN and not self.model.state_specs:
+            self._queued = self._continue_run(run, entries, seed, streams, counters)
+            self.num_runs_queued_ahead += self._queued is not None
+        run.event.synchronize()
+        tokens = self._ring_host_np[run.base:run.base + k, :b].tolist()
+        self.num_graph_replays += run.replays
+        self.num_forward_passes += k
+        self.num_tokens_processed += b * k
+        return tokens
+
+    def _launch_run(self, entries, seed, params, streams, counters, k: int, lookahead: int
+                    ) -> "_QueuedRun":
+        """Upload the batch and queue ``k`` decode steps for it (ring rows ``0..k-1``)."""
+        b = len(entries)
         bucket = 1
         while bucket < b:
             bucket *= 2
         bucket = min(bucket, self.meta.max_seqs)
-        step, _ = self.build_step(entries, pad_to=bucket, lookahead=k - 1)
+        step, _ = self.build_step(entries, pad_to=bucket, lookahead=lookahead)
         # The longest context enters the captured launches only through the number of cuts of
         # the key range, which grows by one per DECODE_KEYS_PER_SPLIT keys up to a limit: graphs
         # are kept per such cell, planned for the cell's lower edge.
@@ -182,11 +220,49 @@ class ModelRunner:
             replays -= 1
         for _ in range(replays):
             graph.graph.replay()
-        self.num_graph_replays += replays
-        tokens = self._run_ring[:k, :b].tolist()
-        self.num_forward_passes += k
-        self.num_tokens_processed += b * k
-        return tokens
+        return self._queue_read(ids, [e.start_pos for e in entries], k, 0, bucket, replays)
+
+    def _queue_read(self, ids, begins, k: int, base: int, bucket: int, replays: int
+                    ) -> "_QueuedRun":
+        """Queue the copy of ring rows ``base..base+k-1`` to the host behind the run's launches."""
+        self._ring_host[base:base + k].copy_(self._run_ring[base:base + k], non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return _QueuedRun(ids, begins, k, base, bucket, replays, event)
+
+    def _continue_run(self, run: "_QueuedRun", entries, seed, streams, counters
+                      ) -> "_QueuedRun | None":
+        """Queue the run that follows ``run`` for the same batch, whose inputs the device holds
+        already; ``None`` where its launches are not captured yet or its pages are missing."""
+        k, cap = run.k, self.meta.max_seqs
+        starts = [p + k for p in run.begins]     # where the following run begins
+        if any(s + k > self.max_model_len for s in starts):
+            return None
+        ctx_bucket = min((max(starts) + 1) // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
+        graph = self.graphs.get((run.bucket, ctx_bucket))
+        if graph is None:
+            return None
+        base = k if run.base == 0 else 0
+        # its pages have to be in the requests' tables by now; they travel behind the launches
+        # that are queued already
+        groups = range(len(self.model.cache_groups))
+        for e, s in zip(entries, starts):
+            if any(len(self.cache.block_table(e.request_id, g)) * self.block_size < s + k for g in groups):
+                return None
+        extend_tables(self.meta, entries, run.bucket, [s + k for s in starts], self.cache.block_table,
+                      self.block_size, self._windowed, self.cache.serial)
+        if self._sample_drawn:
+            fh = self._sample_f_np
+            lo = (2 + base) * cap
+            for i in self._sample_drawn:
+                for j in range(k):
+                    fh[lo + j * cap + i] = uniform(seed, streams[i], counters[i] + k + j)
+            self._sample_f[lo:lo + k * cap].copy_(self._sample_f_host[lo:lo + k * cap], non_blocking=True)
+        if base == 0:
+            self._run_counter.zero_()
+        for _ in range(k):
+            graph.graph.replay()
+        return self._queue_read(run.ids, starts, k, base, run.bucket, k)
 
     def _forward_and_sample(self, step: Step, rows: int) -> torch.Tensor:
         cap = self.meta.max_seqs
@@ -214,6 +290,16 @@ class ModelRunner:
 
 GRAPH_MAX_BATCH = 128  # beyond this the matrix products leave the weight-streaming kernel
 MAX_DECODE_RUN = 16    # decode steps the device can take by itself before the host looks
+
+
+class _QueuedRun:
+    """Decode steps that are queued on the device: whose they are, the position each request
+    begins them at, which ring rows hold their tokens, and the event behind the copy of those
+    rows."""
+
+    def __init__(self, ids, begins, k, base, bucket, replays, event) -> None:
+        self.ids, self.begins, self.k, self.base = ids, begins, k, base
+        self.bucket, self.replays, self.event = bucket, replays, event
 
 
 class _DecodeGraph:

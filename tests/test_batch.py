@@ -7,7 +7,8 @@ import pytest
 import torch
 
 from kvforge_amd.cache import CacheGroup, CacheManager
-from kvforge_amd.engine.batch import MetaBuffers, Step, StepEntry, Workspace, fill_step
+from kvforge_amd.engine.batch import (MetaBuffers, Step, StepEntry, Workspace, extend_tables,
+                                      fill_step)
 
 
 def setup(num_blocks=16, bs=4, groups=None):
@@ -93,6 +94,34 @@ def test_tables_carry_the_pages_of_a_run_of_decode_steps():
     assert step.ctx_lens.tolist() == [4, 0]
     assert not cache.can_append_all([("a", 4 * 16 + 1)])   # more pages than the pool has
     assert step.take_owed(torch.zeros(1)) is None
+
+
+def test_tables_are_extended_without_touching_the_batch():
+    """``extend_tables``: a batch that is on the device keeps its tokens, positions and lengths
+    (the device has moved them on by itself); only its table rows grow."""
+    cache, meta, step = setup()
+    cache.allocate("a", 4)
+    cache.allocate("b", 2)
+    entries = [StepEntry("a", [7], 3, "last"), StepEntry("b", [9], 1, "last")]
+    fill_step(step, meta, entries, cache.block_table, lambda r: -1, 4, pad_to=4)
+    before = meta.device_buf.clone()
+    meta.view("ctx_lens", 4)[:2] += 3            # what the device did meanwhile
+    meta.view("token_ids", 4)[:2] = torch.tensor([55, 66], dtype=torch.int32)
+    cache.append_slots("a", 11, 3)               # two more pages for a, none for b
+    extend_tables(meta, entries, 4, [11, 2], cache.block_table, 4)
+    assert step.block_tables[0][0, :3].tolist() == cache.block_table("a")
+    assert step.block_tables[0][1, :1].tolist() == cache.block_table("b")
+    assert step.block_tables[0][2:].eq(-1).all()
+    assert meta.view("ctx_lens", 4).tolist() == [7, 5, 0, 0]
+    assert meta.view("token_ids", 4)[:2].tolist() == [55, 66]
+    first_table = meta.table_off[0]
+    untouched = torch.ones(meta.total, dtype=torch.bool)
+    untouched[first_table:] = False
+    untouched[meta.off["ctx_lens"]:meta.off["ctx_lens"] + 2] = False
+    untouched[meta.off["token_ids"]:meta.off["token_ids"] + 2] = False
+    assert torch.equal(meta.device_buf[untouched], before[untouched])
+    with pytest.raises(ValueError, match="pages"):
+        extend_tables(meta, entries, 4, [11, 9], cache.block_table, 4)
 
 
 def test_refusals():

@@ -290,6 +290,62 @@ def test_runs_of_decode_steps_on_the_device_equal_single_steps(model_b, dtype):
     assert engine.cache.num_free_blocks == engine.cache.num_blocks
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
+    """While decode runs follow each other for the same requests the next run is queued before
+    the current one is read.  Whatever ends that (a length reached, a stop token, a request that
+    arrives, one that is aborted), the tokens are those of an engine that never queues ahead, no
+    page is lost, and runs were in fact queued and read."""
+    folder, _ = model_b
+    prompts = prompts_for(384, 4, 33, 3, 40)
+    params = [SamplingParams(max_tokens=70, temperature=0.0),
+              SamplingParams(max_tokens=41, temperature=0.9, top_k=40, top_p=0.95, seed=3),
+              SamplingParams(max_tokens=64, temperature=0.0),
+              SamplingParams(max_tokens=23, temperature=1.0, seed=4)]
+
+    def scenario(engine, stop=None):
+        """Two requests; a third arrives after a few steps, a fourth later and is aborted."""
+        ps = list(params)
+        if stop is not None:
+            ps[0] = SamplingParams(max_tokens=70, temperature=0.0, stop_token_ids=[stop])
+        ids = [engine.add_request(prompts[0], ps[0]), engine.add_request(prompts[1], ps[1])]
+        outs, steps = {}, 0
+        while engine.has_unfinished_requests():
+            for o in engine.step():
+                outs[o.request_id] = o
+            steps += 1
+            if steps == 3:
+                ids.append(engine.add_request(prompts[2], ps[2]))
+            if steps == 5:
+                ids.append(engine.add_request(prompts[3], ps[3]))
+            if steps == 7:
+                engine.abort_request(ids[3])
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+        return [(outs[i].output_token_ids, outs[i].finish_reason) for i in ids[:3]]
+
+    for run in (4, 8):
+        plain_engine = engine_for(folder, dtype, decode_run_steps=run, decode_run_ahead=False, seed=2)
+        want = scenario(plain_engine)
+        assert plain_engine.runner.num_runs_queued_ahead == 0
+        engine = engine_for(folder, dtype, decode_run_steps=run, decode_run_ahead=True, seed=2)
+        got = scenario(engine)
+        assert got == want
+        assert engine.runner.num_runs_read_ahead >= 2
+        assert engine.runner.num_runs_queued_ahead > engine.runner.num_runs_read_ahead  # some were left unread
+    # a stop token met while the next run is queued already
+    stop = want[0][0][37]
+    cut = want[0][0].index(stop)
+    engine = engine_for(folder, dtype, decode_run_steps=8, decode_run_ahead=True, seed=2)
+    got = scenario(engine, stop)
+    assert got[0] == (want[0][0][:cut + 1], "stop")
+    plain_stop = scenario(engine_for(folder, dtype, decode_run_steps=8, decode_run_ahead=False, seed=2), stop)
+    assert got == plain_stop
+    # more steps in a run than half the ring holds: nothing is queued ahead
+    engine = engine_for(folder, dtype, decode_run_steps=16, decode_run_ahead=True, seed=2)
+    scenario(engine)
+    assert engine.runner.num_runs_queued_ahead == 0
+
+
 def test_rejections_at_the_entry_point(model_a):
     folder, _ = model_a
     engine = engine_for(folder)
