@@ -450,8 +450,9 @@ int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int 
   }
   if (MT == 1) {
     // Every workgroup reads all of A, so with several rows of A and many rows of W a workgroup
-    // takes 32 rows of W and halves that traffic.
-    const int rw = g_rows_override > 0 ? g_rows_override : (M - m_base > 4 && tiles >= 512 ? 32 : 16);
+    // takes 32 rows of W and halves that traffic; fp32 rows weigh twice as much and make it pay
+    // with fewer rows of W.
+    const int rw = g_rows_override > 0 ? g_rows_override : (M - m_base > 4 && tiles >= (AT ? 256 : 512) ? 32 : 16);
     if (rw == 32) return launch_one<1, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
     if (rw == 64) return launch_one<1, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
   }
