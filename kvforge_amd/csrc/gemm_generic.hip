@@ -79,10 +79,77 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const TA* __restrict__ A
   }
 }
 
+// Few rows of A (decode steps): a tile of 64 x 64 outputs would leave N / 64 workgroups to stream
+// all of W.  Here a workgroup owns 16 columns and 16 rows, one output per thread, and walks K in
+// steps of 64 through LDS; every output is still accumulated over k = 0..K-1 in that order by
+// one thread with the same fused multiply-adds, so it has the same bits as from the kernel above.
+constexpr int RN = 16, RM = 16, RK = 64;
+
+template <typename TA, typename TW, typename TO, int MODE>
+__global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A,
+                                                        const TW* __restrict__ W,
+                                                        TO* __restrict__ C, int M, int N, int K,
+                                                        int lda, int ldc) {
+  __shared__ __align__(16) float As[RM][RK + 4];  // rows 16 bytes apart in banks: no conflicts
+  __shared__ __align__(16) float Ws[RN][RK + 4];
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.y * RM, n0 = blockIdx.x * RN;
+  const int r = tid / RN, c = tid % RN;          // this thread's output
+  const int lrow = tid / 16, lk = (tid % 16) * 4;  // and what it stages: 4 consecutive k of a row
+  // whole 16-byte loads where both operands are fp32 and every row starts on 16 bytes
+  const bool vec = sizeof(TA) == 4 && sizeof(TW) == 4 && K % 4 == 0 && lda % 4 == 0 &&
+                   reinterpret_cast<uintptr_t>(A) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < K; k0 += RK) {
+    {
+      const int m = m0 + lrow, n = n0 + lrow, k = k0 + lk;
+      if (vec) {
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f), w = a;
+        if (m < M && k < K) a = *reinterpret_cast<const float4*>(A + static_cast<size_t>(m) * lda + k);
+        if (n < N && k < K) w = *reinterpret_cast<const float4*>(W + static_cast<size_t>(n) * K + k);
+        *reinterpret_cast<float4*>(&As[lrow][lk]) = a;
+        *reinterpret_cast<float4*>(&Ws[lrow][lk]) = w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          As[lrow][lk + e] = (m < M && k + e < K) ? Elem<TA>::load(A + static_cast<size_t>(m) * lda + k + e) : 0.f;
+          Ws[lrow][lk + e] = (n < N && k + e < K) ? Elem<TW>::load(W + static_cast<size_t>(n) * K + k + e) : 0.f;
+        }
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < RK; kk += 4) {
+      const float4 a = *reinterpret_cast<const float4*>(&As[r][kk]);
+      const float4 w = *reinterpret_cast<const float4*>(&Ws[c][kk]);
+      acc = fmaf(a.x, w.x, acc);
+      acc = fmaf(a.y, w.y, acc);
+      acc = fmaf(a.z, w.z, acc);
+      acc = fmaf(a.w, w.w, acc);
+    }
+    __syncthreads();
+  }
+  const int m = m0 + r, n = n0 + c;
+  if (m >= M || n >= N) return;
+  TO* o = C + static_cast<size_t>(m) * ldc + n;
+  if (MODE == 1) {
+    Elem<TO>::store(o, Elem<TO>::load(o) + acc);
+  } else {
+    Elem<TO>::store(o, acc);
+  }
+}
+
 template <typename TA, typename TW, typename TO, int MODE>
 int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
            hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
+  if (M <= 2 * RM) {
+    dim3 rows_grid((N + RN - 1) / RN, (M + RM - 1) / RM);
+    hipLaunchKernelGGL((gemm_rows_kernel<TA, TW, TO, MODE>), rows_grid, dim3(256), 0, s,
+                       static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C), M,
+                       N, K, lda, ldc);
+    return kvf_last_error();
+  }
   dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   hipLaunchKernelGGL((gemm_tile_kernel<TA, TW, TO, MODE>), grid, dim3(256), 0, s,
                      static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C), M,
