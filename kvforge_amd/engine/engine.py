@@ -122,10 +122,14 @@ class InferenceEngine:
     # ----------------------------------------------------------------- step
     def step(self) -> list[RequestOutput]:
         t0 = time.perf_counter()
-        sched = self.scheduler.schedule()
+        # A run that is queued on the device for the running requests is read before anybody new
+        # is admitted: arrivals wait for at most one run, and no queued work is thrown away.
+        running = sorted(self.scheduler.running, key=self.scheduler._key)
+        queued = self.runner.queued_run_steps([(r.request_id, r.num_computed_tokens) for r in running])
+        sched = self.scheduler.schedule(admit=not queued)
         if sched.is_empty:
             return []
-        run, ahead = self._decode_run_length(sched)
+        run, ahead = self._decode_run_length(sched, queued)
         new_tokens = self._run(sched.scheduled, run, ahead)
         outputs = self._postprocess(sched.scheduled, new_tokens)
         self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens * run,
@@ -133,32 +137,40 @@ class InferenceEngine:
                                  1.0 - self.cache.num_free_blocks / max(1, self.cache.num_blocks))
         return outputs
 
-    def _decode_run_length(self, sched) -> tuple[int, bool]:
+    def _decode_run_length(self, sched, queued: int = 0) -> tuple[int, bool]:
         """How many decode steps the device takes before the host looks again: more than one
         only while every scheduled request decodes, nobody waits for admission, no request can
         reach its length limit inside the run, and the pages of the run's positions are free.
+        ``queued``: the steps of a run that is queued for these requests already (its room and
+        pages were made sure of then).
         The second value says that all of this also holds for the run after it, whose pages are
         then allocated as well, so that the runner may queue that run before this one is read
         (``EngineConfig.decode_run_ahead``)."""
         limit = self.config.decode_run_steps
         group = sched.scheduled
-        if (limit <= 1 or sched.preempted or self.scheduler.num_waiting
-                or any(s.is_prefill or s.num_new_tokens != 1 for s in group)):
+        decoding = not (sched.preempted or any(s.is_prefill or s.num_new_tokens != 1 for s in group))
+        if queued and not decoding:
+            queued = 0  # cannot be: a queued run is for requests that decode
+        if not queued and (limit <= 1 or not decoding or self.scheduler.num_waiting):
             return 1, False
         max_len = self.config.scheduler.max_model_len
         room = min(min(s.request.sampling_params.max_tokens - s.request.num_output_tokens,
                        max_len - s.request.num_tokens) for s in group)
-        limit = min(limit, room)
-        if limit <= 1:
-            return 1, False
-        entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
-                   for s in group]
-        if not self.runner.graph_takes(entries, len(entries)):
-            return 1, False
+        if queued:
+            limit = queued
+        else:
+            limit = min(limit, room)
+            if limit <= 1:
+                return 1, False
+            entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
+                       for s in group]
+            if not self.runner.graph_takes(entries, len(entries)):
+                return 1, False
         wanted = [(s.request.request_id, s.request.num_computed_tokens + limit) for s in group]
-        if not self.cache.can_append_all(wanted):
+        if not queued and not self.cache.can_append_all(wanted):
             return 1, False
-        ahead = self.config.decode_run_ahead and limit == self.config.decode_run_steps and room >= 2 * limit
+        ahead = (self.config.decode_run_ahead and not self.scheduler.num_waiting
+                 and limit == self.config.decode_run_steps and room >= 2 * limit)
         if ahead:
             further = [(rid, total + limit) for rid, total in wanted]
             ahead = self.cache.can_append_all(further)

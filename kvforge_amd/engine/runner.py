@@ -156,23 +156,49 @@ class ModelRunner:
         if not self.graph_takes(entries, len(params)):
             raise ValueError("a decode run takes single tokens that each want their logits")
         queued, self._queued = self._queued, None
-        ids = [e.request_id for e in entries]
-        if (queued is not None and queued.ids == ids and queued.k == k
-                and queued.begins == [e.start_pos for e in entries]):
+        rows = self._rows_in(queued, [(e.request_id, e.start_pos) for e in entries], k)
+        if rows is not None:
             run = queued
             self.num_runs_read_ahead += 1
         else:
             run = self._launch_run(entries, seed, params, streams, counters, k,
                                    lookahead=(2 * k if ahead else k) - 1)
-        if ahead and 2 * k <= MAX_DECODE_RUN and not self.model.state_specs:
+            rows = list(range(b))
+        # Only the whole batch is carried on: rows of requests that have left meanwhile would go
+        # on writing into pages that are no longer theirs.
+        whole = rows == list(range(len(run.ids)))
+        if ahead and whole and 2 * k <= MAX_DECODE_RUN and not self.model.state_specs:
             self._queued = self._continue_run(run, entries, seed, streams, counters)
             self.num_runs_queued_ahead += self._queued is not None
         run.event.synchronize()
-        tokens = self._ring_host_np[run.base:run.base + k, :b].tolist()
+        tokens = self._ring_host_np[run.base:run.base + k][:, rows].tolist()
         self.num_graph_replays += run.replays
         self.num_forward_passes += k
         self.num_tokens_processed += b * k
         return tokens
+
+    @staticmethod
+    def _rows_in(queued: "_QueuedRun | None", wanted: list[tuple[str, int]], k: int
+                 ) -> list[int] | None:
+        """The rows of a queued run that hold the tokens of ``wanted`` (request id, position it
+        begins at), in that order; ``None`` unless every one of them is in the run, in the run's
+        order, at that position, for ``k`` steps.  Requests of the run that are not wanted any
+        more (finished, aborted) are simply not read."""
+        if queued is None or queued.k != k or not wanted:
+            return None
+        place = {rid: i for i, rid in enumerate(queued.ids)}
+        rows = [place.get(rid, -1) for rid, _ in wanted]
+        if any(r < 0 for r in rows) or rows != sorted(rows):
+            return None
+        if any(queued.begins[r] != pos for r, (_, pos) in zip(rows, wanted)):
+            return None
+        return rows
+
+    def queued_run_steps(self, wanted: list[tuple[str, int]]) -> int:
+        """How many steps a run that is queued ahead holds for exactly these requests at these
+        positions (0 if none is queued for them)."""
+        q = self._queued
+        return q.k if q is not None and self._rows_in(q, wanted, q.k) is not None else 0
 
     def _launch_run(self, entries, seed, params, streams, counters, k: int, lookahead: int
                     ) -> "_QueuedRun":

@@ -303,20 +303,27 @@ def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
               SamplingParams(max_tokens=64, temperature=0.0),
               SamplingParams(max_tokens=23, temperature=1.0, seed=4)]
 
+    # In fp32 a token does not depend on what else is in its batch, so requests may arrive while
+    # others decode (with runs queued ahead they are admitted one run later); in bf16 the
+    # batches have to be the same with and without queueing, so all requests are there at once.
+    arrivals = dtype == "float32"
+
     def scenario(engine, stop=None):
         """Two requests; a third arrives after a few steps, a fourth later and is aborted."""
         ps = list(params)
         if stop is not None:
             ps[0] = SamplingParams(max_tokens=70, temperature=0.0, stop_token_ids=[stop])
         ids = [engine.add_request(prompts[0], ps[0]), engine.add_request(prompts[1], ps[1])]
+        if not arrivals:
+            ids += [engine.add_request(prompts[2], ps[2]), engine.add_request(prompts[3], ps[3])]
         outs, steps = {}, 0
         while engine.has_unfinished_requests():
             for o in engine.step():
                 outs[o.request_id] = o
             steps += 1
-            if steps == 3:
+            if steps == 3 and arrivals:
                 ids.append(engine.add_request(prompts[2], ps[2]))
-            if steps == 5:
+            if steps == 5 and arrivals:
                 ids.append(engine.add_request(prompts[3], ps[3]))
             if steps == 7:
                 engine.abort_request(ids[3])
@@ -330,8 +337,8 @@ def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
         engine = engine_for(folder, dtype, decode_run_steps=run, decode_run_ahead=True, seed=2)
         got = scenario(engine)
         assert got == want
-        assert engine.runner.num_runs_read_ahead >= 2
-        assert engine.runner.num_runs_queued_ahead > engine.runner.num_runs_read_ahead  # some were left unread
+        # every queued run was read: by all of its requests, or by those that were left
+        assert engine.runner.num_runs_read_ahead == engine.runner.num_runs_queued_ahead >= 3
     # a stop token met while the next run is queued already
     stop = want[0][0][37]
     cut = want[0][0].index(stop)

@@ -75,6 +75,22 @@ def test_decodes_are_scheduled_before_new_prefills():   # :70-77
     assert [x.request.request_id for x in out.prefills] == ["b"]
 
 
+def test_a_step_without_admission_leaves_arrivals_waiting():
+    """``schedule(admit=False)`` (the engine's step that reads decode steps already queued on the
+    device): the running request decodes, the arrival waits one step and is admitted the next."""
+    s = make()
+    s.add_request(req("a", 4, 1.0))
+    complete(s.schedule())
+    s.add_request(req("b", 4, 2.0))
+    out = s.schedule(admit=False)
+    assert [(x.request.request_id, x.num_new_tokens, x.is_prefill) for x in out.scheduled] == [("a", 1, False)]
+    assert s.num_waiting == 1 and s.num_running == 1
+    complete(out)
+    out = s.schedule()
+    assert [(x.request.request_id, x.is_prefill) for x in out.scheduled] == [("a", False), ("b", True)]
+    assert s.num_waiting == 0
+
+
 def test_rejections():                             # :80-89 and scheduler.py:109-129
     s = make(max_num_batched_tokens=8, enable_chunked_prefill=False)
     with pytest.raises(RequestRejectedError):
