@@ -132,15 +132,17 @@ class InferenceEngine:
         run, ahead = self._decode_run_length(sched, queued)
         new_tokens = self._run(sched.scheduled, run, ahead)
         outputs = self._postprocess(sched.scheduled, new_tokens)
-        self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens * run,
-                                 time.perf_counter() - t0,
-                                 1.0 - self.cache.num_free_blocks / max(1, self.cache.num_blocks))
+        # a run of decode steps counts as that many steps of the batch, each with its share of the time
+        dt = (time.perf_counter() - t0) / run
+        used = 1.0 - self.cache.num_free_blocks / max(1, self.cache.num_blocks)
+        for _ in range(run):
+            self.metrics.record_step(len(sched.scheduled), sched.num_batched_tokens, dt, used)
         return outputs
 
     def _decode_run_length(self, sched, queued: int = 0) -> tuple[int, bool]:
         """How many decode steps the device takes before the host looks again: more than one
         only while every scheduled request decodes, nobody waits for admission, no request can
-        reach its length limit inside the run, and the pages of the run's positions are free.
+        reach the model's length inside the run, and the pages of the run's positions are free.
         ``queued``: the steps of a run that is queued for these requests already (its room and
         pages were made sure of then).
         The second value says that all of this also holds for the run after it, whose pages are
@@ -153,13 +155,16 @@ class InferenceEngine:
             queued = 0  # cannot be: a queued run is for requests that decode
         if not queued and (limit <= 1 or not decoding or self.scheduler.num_waiting):
             return 1, False
+        # A request that reaches its number of tokens inside a run is cut there when the run is
+        # read, like one that meets a stop token; only the model's length is a hard limit.  No
+        # run is longer than the longest remainder.
         max_len = self.config.scheduler.max_model_len
-        room = min(min(s.request.sampling_params.max_tokens - s.request.num_output_tokens,
-                       max_len - s.request.num_tokens) for s in group)
+        room = min(max_len - s.request.num_tokens for s in group)
+        longest = max(s.request.sampling_params.max_tokens - s.request.num_output_tokens for s in group)
         if queued:
             limit = queued
         else:
-            limit = min(limit, room)
+            limit = min(limit, room, longest)
             if limit <= 1:
                 return 1, False
             entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
@@ -170,7 +175,7 @@ class InferenceEngine:
         if not queued and not self.cache.can_append_all(wanted):
             return 1, False
         ahead = (self.config.decode_run_ahead and not self.scheduler.num_waiting
-                 and limit == self.config.decode_run_steps and room >= 2 * limit)
+                 and limit == self.config.decode_run_steps and room >= 2 * limit and longest > limit)
         if ahead:
             further = [(rid, total + limit) for rid, total in wanted]
             ahead = self.cache.can_append_all(further)
