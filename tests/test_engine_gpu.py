@@ -353,6 +353,54 @@ def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
     assert engine.runner.num_runs_queued_ahead == 0
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
+    """Requests of random lengths arrive at random steps into a pool so small that some are
+    preempted; some carry stop tokens, two are aborted.  In fp32 a token does not depend on its
+    batch, so every way of running (single steps, runs, runs queued ahead) must give every
+    request the same tokens and the same end, and give every page back."""
+    folder, _ = model_a
+    rng = random.Random(seed)
+    n = 12
+    prompts = prompts_for(256, n, 100 + seed, 1, 30)
+    params = [SamplingParams(max_tokens=rng.randint(1, 40), temperature=rng.choice([0.0, 0.0, 0.8]),
+                             top_k=rng.choice([0, 20]), seed=7,
+                             stop_token_ids=rng.sample(range(256), rng.choice([0, 0, 12])))
+              for _ in range(n)]
+    arrive = sorted(rng.randint(0, 25) for _ in range(n))
+    aborted = {rng.randrange(n): rng.randint(3, 30), rng.randrange(n): rng.randint(3, 30)}
+
+    def run(**kw):
+        engine = engine_for(folder, "float32", block_size=4, num_blocks=40, max_num_seqs=6,
+                            max_num_batched_tokens=32, seed=5, **kw)
+        ids, outs, step = {}, {}, 0
+        while len(ids) < n or engine.has_unfinished_requests():
+            for i in range(n):
+                if i not in ids and arrive[i] <= step:
+                    ids[i] = engine.add_request(prompts[i], params[i])
+            for i, when in aborted.items():
+                if when == step and i in ids:
+                    engine.abort_request(ids[i])
+            for o in engine.step():
+                outs[o.request_id] = o
+            step += 1
+            assert step < 2000
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+        return ({i: (outs[ids[i]].output_token_ids, outs[ids[i]].finish_reason)
+                 for i in range(n) if i not in aborted and ids[i] in outs}, engine)
+
+    want, single = run(decode_run_steps=1)
+    assert len(want) >= n - 2
+    saw_ahead = 0
+    for kw in (dict(decode_run_steps=8, decode_run_ahead=False), dict(decode_run_steps=8, decode_run_ahead=True),
+               dict(decode_run_steps=3, decode_run_ahead=True)):
+        got, engine = run(**kw)
+        assert got == want, kw
+        saw_ahead += engine.runner.num_runs_read_ahead
+    assert single.scheduler.num_preemptions > 0 or seed != 0   # the pool is meant to run out
+    assert saw_ahead > 0                                        # and runs are meant to be queued ahead
+
+
 def test_rejections_at_the_entry_point(model_a):
     folder, _ = model_a
     engine = engine_for(folder)
