@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--prompt-len 512]
                     [--dtype bfloat16] [--layers L] [--no-points] [--phase all|decode|prefill]
                     [--preset llama-1b|llama-3b|llama-8b] [--context-len 8192]
+    python bench.py --phase mixed --preset llama-3b --batch 32 --steps 256
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -127,6 +128,28 @@ def prefill_run(engine, vocab, tokens, repeats=3, seed=1):
     return best
 
 
+def mixed_run(engine, vocab, requests, new_tokens, seed=0):
+    """``requests`` prompts of 128 to 4,096 tokens (uniform), all there at once: chunked prefill
+    under the token budget mixed with the decode steps of those already running, ``new_tokens``
+    each.  Returns prompt tokens, generated tokens and seconds."""
+    import random
+    import torch
+    from kvforge_amd import SamplingParams
+
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    lens = [rng.randint(128, 4096) for _ in range(requests)]
+    prompts = [torch.randint(1, vocab, (n,), generator=g).tolist() for n in lens]
+    params = SamplingParams(max_tokens=new_tokens, temperature=0.0, ignore_eos=True)
+    engine.generate(prompts[:2], SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True))  # warm-up
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    outs = engine.generate(prompts, params)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return sum(lens), sum(len(o.output_token_ids) for o in outs), dt
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -152,8 +175,10 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill"], default="all",
-                    help="for profiles: only the decode steps at --batch, or only the prefill")
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed"], default="all",
+                    help="for profiles: only the decode steps at --batch, or only the prefill; "
+                         "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
+                         "prefill beside decode steps, --steps new tokens each")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -172,6 +197,17 @@ def main() -> int:
 
     with tempfile.TemporaryDirectory(prefix="kvforge_bench_") as folder:
         kvforge_amd.write_random_model(folder, cfg, seed=0)
+        if args.phase == "mixed":
+            engine = build_engine(folder, args.dtype, args.batch, args.batch * (4096 + args.steps + 64),
+                                  use_graphs=not args.no_graphs, run_steps=args.decode_run_steps,
+                                  context_cap=args.context_len)
+            prompt_tokens, generated, dt = mixed_run(engine, vocab, args.batch, args.steps)
+            print(json.dumps({"phase": "mixed", "model": args.preset, "requests": args.batch,
+                              "dtype": args.dtype, "prompt_tokens": prompt_tokens,
+                              "generated_tokens": generated, "seconds": round(dt, 4),
+                              "total_tok_s": round((prompt_tokens + generated) / dt, 1),
+                              "generated_tok_s": round(generated / dt, 1)}))
+            return 0
         results = {}
         points = args.phase == "all" and not args.no_points
         batches = [args.batch] + ([b for b in (1, 64) if b != args.batch] if points else [])
