@@ -50,6 +50,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
     p.add_argument("--no-graphs", action="store_true", help="do not replay decode steps from HIP graphs")
     p.add_argument("--decode-run-steps", type=int, default=8,
                    help="decode steps the device takes between two looks of the host")
+    p.add_argument("--no-decode-run-ahead", action="store_true",
+                   help="do not queue the next run of decode steps before the current one is read")
     p.add_argument("--json", action="store_true", help="print one JSON object instead of text")
     return p.parse_args(argv)
 
@@ -80,7 +82,7 @@ def main(argv: list[str] | None = None) -> int:
                                   max_num_batched_tokens=args.max_num_batched_tokens,
                                   max_model_len=args.max_model_len),
         device=args.device, dtype=args.dtype, seed=args.seed, use_graphs=not args.no_graphs,
-        decode_run_steps=args.decode_run_steps)
+        decode_run_steps=args.decode_run_steps, decode_run_ahead=not args.no_decode_run_ahead)
     if args.model:
         engine = InferenceEngine.from_folder(args.model, config, tokenizer)
         name = args.model
