@@ -353,6 +353,43 @@ def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
     assert engine.runner.num_runs_queued_ahead == 0
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_window_layers_give_pages_back_while_runs_go_on(tmp_path, dtype):
+    """Two kinds of layer (all keys; the last 24): pages behind the window go back to the pool
+    while the request lives, also when the device takes runs of steps by itself and the next run
+    is queued before the host has read the current one.  Tokens are the plain model's choices
+    (fp32) and the same however the steps are run."""
+    from tests.replay_util import TINY_C, sharpen
+    folder = str(tmp_path / "c")
+    kvforge_amd.write_random_model(folder, TINY_C, seed=3)
+    sharpen(folder, 6.0)
+    oracle = Oracle(folder)
+    prompts = prompts_for(200, 3, 8, 20, 60)
+    params = SamplingParams(max_tokens=90, temperature=0.0)
+    results = []
+    for kw in (dict(decode_run_steps=1), dict(decode_run_steps=8, decode_run_ahead=False),
+               dict(decode_run_steps=8, decode_run_ahead=True)):
+        engine = engine_for(folder, dtype, block_size=4, num_blocks=160, **kw)
+        ids = [engine.add_request(p, params) for p in prompts]
+        windowed = [g.window is not None for g in engine.cache.groups]
+        assert sorted(windowed) == [False, True]
+        outs, peak = {}, [0, 0]
+        while engine.has_unfinished_requests():
+            for o in engine.step():
+                outs[o.request_id] = o
+            peak = [max(p, pool.num_used) for p, pool in zip(peak, engine.cache.pools)]
+        # the group that keeps every key grows with the requests, the other stays near its window
+        assert peak[windowed.index(True)] < peak[windowed.index(False)] // 2
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+        results.append([outs[i].output_token_ids for i in ids])
+        if kw.get("decode_run_ahead"):
+            assert engine.runner.num_runs_read_ahead > 0
+    assert results[1] == results[0] and results[2] == results[0]
+    if dtype == "float32":
+        for p, out in zip(prompts, results[0]):
+            oracle.check_choices(p, out, 1e-4)
+
+
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
     """Requests of random lengths arrive at random steps into a pool so small that some are
