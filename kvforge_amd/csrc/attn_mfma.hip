@@ -695,6 +695,8 @@ void launch_split_waves(dim3 grid, hipStream_t s, const void* q, const void* k_p
                      static_cast<bf16_t*>(out), part_acc, part_ml, a);
 }
 
+int g_split_waves = 0;  // measurement aid: 4 or 8 waves per workgroup, 0 = by the grid
+
 // Eight waves shorten each wave's walk over the keys when the grid leaves compute units idle
 // anyway (and two blocks of fragments still fit the registers that leaves each wave); a grid
 // that fills the chip does better with four.
@@ -703,7 +705,8 @@ void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, 
                   const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
                   void* out, float* part_acc, float* part_ml, const MArgs& a) {
   const size_t groups = static_cast<size_t>(grid.x) * grid.y * grid.z;
-  if (DT <= 6 && groups <= 256)
+  const bool eight = g_split_waves ? g_split_waves == 8 : groups <= 256;
+  if (DT <= 6 && eight)
     launch_split_waves<DT, (DT <= 6 ? 8 : 4)>(grid, s, q, k_pages, vt_pages, block_table, seq_ids, cu_q,
                                               ctx_lens, out, part_acc, part_ml, a);
   else
@@ -716,6 +719,8 @@ void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, 
 }  // namespace
 
 // Rows of a query run one workgroup takes: 4 waves x RT tiles x 16 rows.
+// For measurements: waves per workgroup of the kernel for single tokens (4, 8; 0 = by the grid).
+KVF_EXPORT void kvf_attn_mfma_set_split_waves(int waves) { g_split_waves = waves; }
 KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d) { return WAVES * runs_rt(d / 16) * 16; }
 
 // Query runs: `work` holds num_work rows (sequence, item, item or -1) where item i covers rows

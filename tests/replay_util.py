@@ -28,6 +28,20 @@ TINY_C = {  # differs from tiny-a and tiny-b in every size; two kinds of attenti
 }
 
 
+WIDE = {  # layers wide enough for the kernels that serving a real model takes: head size 64 on
+    # the matrix cores, a down projection deep and narrow enough to be cut in two halves of K (one
+    # of them stays owed to the stream until the next layer's projections), gate/up wide enough
+    # for two groups of columns per wave, a vocabulary that ends inside a group of 16 columns
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 1000,
+    "hidden_size": 256, "num_hidden_layers": 3, "num_attention_heads": 4, "num_key_value_heads": 2,
+    "head_dim": 64, "intermediate_size": 4096, "max_position_embeddings": 512,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 128},
+    "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": True,
+}
+
+
 def sharpen(folder: str, factor: float) -> None:
     """Scale every q and k projection so that attention is peaked: with N(0, 0.02) weights the
     scores are nearly flat and one misplaced key would hide among hundreds."""

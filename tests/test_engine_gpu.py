@@ -519,6 +519,33 @@ def test_graph_replay_equals_eager_steps(model_b, dtype):
     assert graphed == eager
 
 
+def test_wide_layers_through_graphs_and_queued_runs(tmp_path):
+    """A model whose layers are wide enough for the kernels a real model is served with (the down
+    projection in two halves of K, one of them owed from layer to layer; two groups of columns
+    per wave in gate/up; head size 64 on the matrix cores): six requests in bf16 through captured
+    graphs, runs of steps on the device and runs queued ahead give the tokens of single eager
+    steps, and every token is the plain model's choice within bf16 rounding."""
+    from tests.replay_util import WIDE, sharpen
+    folder = str(tmp_path / "wide")
+    kvforge_amd.write_random_model(folder, dict(WIDE), seed=4)
+    sharpen(folder, 4.0)
+    oracle = Oracle(folder)
+    prompts = prompts_for(1000, 6, 17, 5, 60)
+    params = SamplingParams(max_tokens=40, temperature=0.0)
+
+    def run(**kw):
+        engine = engine_for(folder, "bfloat16", block_size=16, num_blocks=128, max_num_seqs=8,
+                            max_num_batched_tokens=512, **kw)
+        return [o.output_token_ids for o in engine.generate(prompts, params)], engine
+
+    eager, _ = run(use_graphs=False, decode_run_steps=1)
+    served, engine = run(use_graphs=True, decode_run_steps=8, decode_run_ahead=True)
+    assert engine.runner.num_graph_replays > 0 and engine.runner.num_runs_queued_ahead >= 1
+    assert served == eager
+    for p, out in zip(prompts, served):
+        oracle.check_choices(p, out, 3e-2)
+
+
 @pytest.mark.parametrize("count,bucket", [(24, 32), (40, 64)])
 def test_graph_replay_with_many_requests(model_a, count, bucket):
     """Many requests decode together.  A padded batch of 32 is two row tiles of the hand-written

@@ -58,6 +58,27 @@ def test_replay_all_modes(tmp_path, name, dtype, sharp):
     ru.compare(folder, tb, out, names, atol, rtol)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype):
+    """The tiny configurations are below the sizes at which the bf16 engine changes kernels.
+    This one is not: its down projection is cut in two halves of K for up to 16 rows, and the
+    half that stays owed travels to the next layer's fused q/k/v projection and to the final
+    norm; attention runs on the matrix cores at head size 64.  All four ways of cutting the
+    requests, against the plain model."""
+    import torch
+    from kvforge_amd.kernels import ops
+    bf = torch.bfloat16
+    few, deep = torch.empty(3, 4096, dtype=bf), torch.empty(256, 4096, dtype=bf)
+    assert ops.k_halves_pay(few, deep) and not ops.is_library_product(few, deep)
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, dict(ru.WIDE), seed=4)
+    prompts = ru.random_prompts(1000, [41, 75, 52, 66], 9)
+    tb, names = build_all_modes(prompts, 9)
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, dtype, tb, out)
+    ru.compare(folder, tb, out, names, *TOL[dtype])
+
+
 def test_replay_first_tokens_and_one_token_requests(tmp_path):
     """The first tokens of a sequence: a request of one token, of two, a first step of one token
     followed by a portion, and position 0 decoded alone."""
