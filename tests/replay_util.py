@@ -42,6 +42,12 @@ WIDE = {  # layers wide enough for the kernels that serving a real model takes: 
 }
 
 
+# the same with head size 128, one kv head, a width that is not heads x head size, untied head
+WIDE_B = dict(WIDE, vocab_size=777, hidden_size=192, num_hidden_layers=2, num_attention_heads=2,
+              num_key_value_heads=1, head_dim=128, intermediate_size=4608, rms_norm_eps=1e-6,
+              tie_word_embeddings=False)
+
+
 def sharpen(folder: str, factor: float) -> None:
     """Scale every q and k projection so that attention is peaked: with N(0, 0.02) weights the
     scores are nearly flat and one misplaced key would hide among hundreds."""

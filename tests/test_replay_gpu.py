@@ -59,7 +59,8 @@ def test_replay_all_modes(tmp_path, name, dtype, sharp):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype):
+@pytest.mark.parametrize("which", ["WIDE", "WIDE_B"])
+def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, which):
     """The tiny configurations are below the sizes at which the bf16 engine changes kernels.
     This one is not: its down projection is cut in two halves of K for up to 16 rows, and the
     half that stays owed travels to the next layer's fused q/k/v projection and to the final
@@ -68,11 +69,13 @@ def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype):
     import torch
     from kvforge_amd.kernels import ops
     bf = torch.bfloat16
-    few, deep = torch.empty(3, 4096, dtype=bf), torch.empty(256, 4096, dtype=bf)
+    cfg = dict(getattr(ru, which))
+    few = torch.empty(3, cfg["intermediate_size"], dtype=bf)
+    deep = torch.empty(cfg["hidden_size"], cfg["intermediate_size"], dtype=bf)
     assert ops.k_halves_pay(few, deep) and not ops.is_library_product(few, deep)
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, dict(ru.WIDE), seed=4)
-    prompts = ru.random_prompts(1000, [41, 75, 52, 66], 9)
+    kvforge_amd.write_random_model(folder, cfg, seed=4)
+    prompts = ru.random_prompts(cfg["vocab_size"], [41, 75, 52, 66], 9)
     tb, names = build_all_modes(prompts, 9)
     out = str(tmp_path / "out")
     ru.run_trace(folder, dtype, tb, out)
