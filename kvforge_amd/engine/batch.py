@@ -55,9 +55,14 @@ class Workspace:
     def __init__(self, device: torch.device | str) -> None:
         self.device = device
         self._bufs: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+        # views handed out before, by (name, dtype, shape): a step asks for the same ones again
+        self._views: dict[tuple, torch.Tensor] = {}
         self.frozen = False
 
     def buf(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
@@ -68,7 +73,12 @@ class Workspace:
                 raise RuntimeError(f"workspace buffer {name} would grow during graph capture")
             flat = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = flat
-        return flat[:n].view(shape)
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]           # they show the memory that was let go
+        view = flat[:n].view(shape)
+        if len(self._views) < 4096:
+            self._views[(name, dtype, shape)] = view
+        return view
 
     def zeros(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         """Like ``buf`` for memory whose users leave it zero: cleared once, when it is made."""
@@ -82,6 +92,8 @@ class Workspace:
                 raise RuntimeError(f"workspace buffer {name} would grow during graph capture")
             flat = torch.zeros(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = flat
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]
         return flat[:n].view(shape)
 
     def snapshot(self) -> list[torch.Tensor]:

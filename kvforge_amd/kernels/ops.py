@@ -33,7 +33,13 @@ def _suffix(dtype: torch.dtype) -> str:
     return "f32" if _tcode(dtype) == 0 else "bf16"
 
 
+# the raw handle of torch's current stream, without a Stream object built for every launch
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -43,9 +49,15 @@ def _check(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True) 
     if dtype is not None and t.dtype != dtype:
         raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
     if shape is not None:
-        if t.dim() != len(shape) or any(s is not None and int(s) != int(ts)
-                                        for s, ts in zip(shape, t.shape)):
-            raise KernelError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+        have = t.shape
+        bad = len(have) != len(shape)
+        if not bad:
+            for want, got in zip(shape, have):   # a plain loop: this runs for every operand of every launch
+                if want is not None and want != got:
+                    bad = True
+                    break
+        if bad:
+            raise KernelError(f"{name} must have shape {list(shape)}, got {list(have)}")
     if contiguous and not t.is_contiguous():
         raise KernelError(f"{name} must be contiguous")
 
