@@ -32,6 +32,9 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
 # prefill kernel's time).  Masked scores are -inf and no NaN is formed from them (an empty row's
 # reference is replaced by zero before it is subtracted), so the kernel may assume there are none.
 MODULE_FLAGS: dict[str, list[str]] = {"attn_mfma": ["-fno-honor-nans"]}
+# Libraries a module is linked against (after its sources on the command line).
+ROCM_LIB = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
+MODULE_LINK: dict[str, list[str]] = {"gemm_library": [f"-L{ROCM_LIB}", f"-Wl,-rpath,{ROCM_LIB}", "-lhipblaslt"]}
 HEADERS = ["common.h"]
 MODULES: dict[str, list[str]] = {
     "elementwise": ["elementwise.hip"],
@@ -40,6 +43,7 @@ MODULES: dict[str, list[str]] = {
     "attn_generic": ["attn_generic.hip"],
     "attn_mfma": ["attn_mfma.hip"],
     "sampling": ["sampling.hip"],
+    "gemm_library": ["gemm_library.hip"],
 }
 
 
@@ -123,7 +127,7 @@ def build_module(name: str, force: bool = False, verbose: bool = True) -> str:
     out_dir = _build_dir()
     so, stamp = os.path.join(out_dir, f"{name}.so"), os.path.join(out_dir, f"{name}.stamp")
     tmp = os.path.join(out_dir, f".{name}.{os.getpid()}.{threading.get_ident()}.so")
-    cmd = [hipcc, *FLAGS, *MODULE_FLAGS.get(name, []), f"-I{CSRC}", *[os.path.join(CSRC, s) for s in MODULES[name]], "-o", tmp]
+    cmd = [hipcc, *FLAGS, *MODULE_FLAGS.get(name, []), f"-I{CSRC}", *[os.path.join(CSRC, s) for s in MODULES[name]], *MODULE_LINK.get(name, []), "-o", tmp]
     t0 = time.time()
     if verbose:
         _log(f"compiling kernel module {name} for {ARCH} ...")

@@ -8,7 +8,7 @@ There is no fallback: every function here runs a hand-written gfx950 kernel or r
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_float, c_int, c_void_p
+from ctypes import c_float, c_int, c_long, c_void_p
 
 import torch
 
@@ -313,6 +313,39 @@ def k_halves_pay(a: torch.Tensor, w) -> bool:
             and -(-w.shape[0] // 16) <= K_HALVES_MAX_GROUPS)
 
 
+# The library's product is called through an entry point of our own: torch.mm costs 17 us of
+# host time a call, which is what bounds a step that is launched kernel by kernel (a portion of a
+# prompt) at a few hundred rows.  LIBRARY_DIRECT = False sends them through torch.mm again.
+LIBRARY_DIRECT = True
+LIBRARY_WORKSPACE_BYTES = 76 << 20
+_library_ready: dict[int, bool] = {}
+_LIBRARY_ARGS = [c_void_p, c_void_p, c_void_p] + [c_int] * 7 + [c_void_p]
+
+
+def _library_product(a, w, out, accumulate, m, n, k, lda, ldc) -> bool:
+    """``out = a @ w.T`` (or ``+=``, in fp32) by hipBLASLt, with fp32 sums stored as ``out`` has
+    them.  False where that route is closed: switched off, not set up yet while a stream is
+    being captured (its workspace cannot be allocated then), or no algorithm for the shape."""
+    if not LIBRARY_DIRECT or out.dtype not in (F32, BF16) or (accumulate and out.dtype != F32):
+        return False
+    dev = a.device.index if a.device.index is not None else torch.cuda.current_device()
+    ready = _library_ready.get(dev)
+    if ready is None:
+        if torch.cuda.is_current_stream_capturing():
+            return False
+        init = _fn("gemm_library", "kvf_gemm_library_init", [c_long])
+        with torch.cuda.device(dev):
+            _ok(init(LIBRARY_WORKSPACE_BYTES), "gemm_library_init")
+        ready = _library_ready[dev] = True
+    f = _fn("gemm_library", "kvf_gemm_library_bf16", _LIBRARY_ARGS)
+    code = f(a.data_ptr(), w.data_ptr(), out.data_ptr(), 1 if out.dtype == F32 else 0,
+             1 if accumulate else 0, m, n, k, lda, ldc, _stream())
+    if code == -1:
+        return False
+    _ok(code, "gemm_library")
+    return True
+
+
 def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
          owed: torch.Tensor | None = None, half_out: torch.Tensor | None = None) -> None:
     """``out = a @ w.T`` (``accumulate``: ``out += a @ w.T`` with ``out`` fp32).
@@ -353,6 +386,8 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
             return
         if owed is not None:
             out.add_(owed)
+        if _library_product(a, plain_of(w), out, accumulate, m, n, k, lda, ldc):
+            return
         if accumulate:
             # many rows: the library's bf16 product, then the residual sum in fp32
             out.add_(torch.mm(a, plain_of(w).t()))
