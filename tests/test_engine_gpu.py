@@ -519,6 +519,32 @@ def test_graph_replay_equals_eager_steps(model_b, dtype):
     assert graphed == eager
 
 
+def test_graph_replay_of_library_products_at_the_served_width(tmp_path):
+    """64 requests decode through layers of the Llama 3.2 1B shape (two of them, and a small
+    vocabulary, to keep the folder small): a padded batch of 64 rows sends every product to the
+    library, whose kernels for these widths (up to 16,384 columns, K up to 8,192) are others than
+    the tiny models meet and may bring a workspace along.  Replays of the captured graph, with
+    eager prefill steps and synchronisations around them, give the tokens of eager launches."""
+    cfg = kvforge_amd.preset_dict("llama-1b")
+    cfg.update(num_hidden_layers=2, vocab_size=4096)
+    folder = str(tmp_path / "served")
+    kvforge_amd.write_random_model(folder, cfg, seed=0)
+    prompts = prompts_for(4096, 64, 5, 8, 40)
+    params = SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True)
+
+    def run(use_graphs):
+        engine = engine_for(folder, "bfloat16", block_size=16, num_blocks=512, max_num_seqs=64,
+                            max_num_batched_tokens=4096, use_graphs=use_graphs)
+        return [o.output_token_ids for o in engine.generate(prompts, params)], engine
+
+    eager, _ = run(False)
+    graphed, engine = run(True)
+    assert any(b == 64 for b, _ in engine.runner.graphs) and engine.runner.num_graph_replays >= 16
+    assert graphed == eager
+    again, _ = run(True)
+    assert again == graphed
+
+
 def test_wide_layers_through_graphs_and_queued_runs(tmp_path):
     """A model whose layers are wide enough for the kernels a real model is served with (the down
     projection in two halves of K, one of them owed from layer to layer; two groups of columns
