@@ -141,8 +141,12 @@ class InferenceEngine:
 
     def _decode_run_length(self, sched, queued: int = 0) -> tuple[int, bool]:
         """How many decode steps the device takes before the host looks again: more than one
-        only while every scheduled request decodes, nobody waits for admission, no request can
-        reach the model's length inside the run, and the pages of the run's positions are free.
+        only while every scheduled request decodes, no request can reach the model's length
+        inside the run, and the pages of the run's positions are free.  While requests wait
+        that the scheduler could not admit beside these (no sequence slot, no pages), nothing
+        changes for them before a running request ends: the run then goes up to the first end
+        that is certain, the smallest number of tokens a request has left (one that meets a
+        stop token earlier keeps its slot until the run is read).
         ``queued``: the steps of a run that is queued for these requests already (its room and
         pages were made sure of then).
         The second value says that all of this also holds for the run after it, whose pages are
@@ -153,18 +157,19 @@ class InferenceEngine:
         decoding = not (sched.preempted or any(s.is_prefill or s.num_new_tokens != 1 for s in group))
         if queued and not decoding:
             queued = 0  # cannot be: a queued run is for requests that decode
-        if not queued and (limit <= 1 or not decoding or self.scheduler.num_waiting):
+        if not queued and (limit <= 1 or not decoding):
             return 1, False
         # A request that reaches its number of tokens inside a run is cut there when the run is
         # read, like one that meets a stop token; only the model's length is a hard limit.  No
         # run is longer than the longest remainder.
         max_len = self.config.scheduler.max_model_len
         room = min(max_len - s.request.num_tokens for s in group)
-        longest = max(s.request.sampling_params.max_tokens - s.request.num_output_tokens for s in group)
+        left = [s.request.sampling_params.max_tokens - s.request.num_output_tokens for s in group]
+        longest = max(left)
         if queued:
             limit = queued
         else:
-            limit = min(limit, room, longest)
+            limit = min(limit, room, min(left) if self.scheduler.num_waiting else longest)
             if limit <= 1:
                 return 1, False
             entries = [StepEntry(s.request.request_id, [0], s.request.num_computed_tokens, "last")
