@@ -290,6 +290,34 @@ def test_runs_of_decode_steps_on_the_device_equal_single_steps(model_b, dtype):
     assert engine.cache.num_free_blocks == engine.cache.num_blocks
 
 
+def test_runs_go_on_while_blocked_requests_wait(model_a):
+    """Six requests over two sequence slots: those that wait cannot be admitted before a running
+    one ends, so the device keeps taking steps by itself up to the first end that is certain (the
+    fewest tokens left), and the slot is filled in the very next step, as with single steps:
+    same tokens, same number of model steps, far fewer looks of the host."""
+    folder, oracle = model_a
+    prompts = prompts_for(256, 6, 8, 3, 12)
+    params = [SamplingParams(max_tokens=n, temperature=0.0) for n in (20, 9, 17, 12, 25, 6)]
+
+    def run(steps):
+        engine = engine_for(folder, "float32", max_num_seqs=2, decode_run_steps=steps)
+        ids = [engine.add_request(p, sp) for p, sp in zip(prompts, params)]
+        outs, looks = {}, 0
+        while engine.has_unfinished_requests():
+            for o in engine.step():
+                outs[o.request_id] = o.output_token_ids
+            looks += 1
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+        return [outs[i] for i in ids], looks, engine
+
+    want, single_looks, single = run(1)
+    got, looks, engine = run(8)
+    assert got == want and [len(t) for t in got] == [20, 9, 17, 12, 25, 6]
+    assert engine.runner.num_forward_passes == single.runner.num_forward_passes
+    assert looks < single_looks // 2
+    oracle.check_choices(prompts[4], got[4], 1e-4)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_runs_queued_ahead_give_the_same_tokens(model_b, dtype):
     """While decode runs follow each other for the same requests the next run is queued before
