@@ -105,14 +105,6 @@ KVF_EXPORT int kvf_gemm_library_init(long workspace_bytes) {
   return 0;
 }
 
-// 1 once kvf_gemm_library_init has run for the current device.
-KVF_EXPORT int kvf_gemm_library_ready() {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 0;
-  std::lock_guard<std::mutex> hold(g_lock);
-  return g_dev[dev].handle ? 1 : 0;
-}
-
 // C = A * W^T (accumulate: C += A * W^T; fp32 C only).  A: bf16 [M, K], row stride lda; W: bf16
 // [N, K] contiguous; C: [M, N] bf16 or fp32 (out_f32), row stride ldc.  Returns 0, a HIP error
 // code, or -1 where the library offers no algorithm for the shape (the caller takes another
