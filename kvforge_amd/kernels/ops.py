@@ -277,6 +277,12 @@ def _gemm_operands(a, w, out, n_out):
     return m, n, k, lda, ldc
 
 
+def _rows_aligned(a: torch.Tensor, k: int, lda: int) -> bool:
+    """Rows that the matrix-core kernels (and the library) read 16 bytes at a time: eight
+    elements per step of K, every row and the first one at a multiple of 16 bytes."""
+    return k % 8 == 0 and lda % 8 == 0 and a.data_ptr() % 16 == 0
+
+
 def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False,
                       fused_epilogue: bool = False) -> bool:
     """Whether the MFMA weight-streaming kernel takes these operands: bf16 weights, bf16 rows
@@ -288,7 +294,7 @@ def bf16_kernel_takes(a: torch.Tensor, w: torch.Tensor, rms: bool = False,
     m, k = a.shape
     lda = a.stride(0) if m > 1 else k
     limit = FUSED_NORM_MAX_M if rms else (FUSED_EPILOGUE_MAX_M if fused_epilogue else SKINNY_MAX_M)
-    return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and k % 8 == 0 and lda % 8 == 0
+    return (w.dtype == BF16 and a.dtype == (F32 if rms else BF16) and _rows_aligned(a, k, lda)
             and m <= limit)
 
 
@@ -300,7 +306,7 @@ def is_library_product(a: torch.Tensor, w: torch.Tensor) -> bool:
     m, k = a.shape
     n = w.shape[0]
     lda = a.stride(0) if m > 1 else k
-    return (a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0
+    return (a.dtype == BF16 and w.dtype == BF16 and _rows_aligned(a, k, lda)
             and (m > SKINNY_MAX_M or (m > 16 and k >= 2 * n)))
 
 
@@ -376,7 +382,7 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
     out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)
     if not accumulate:
         _tcode(out.dtype)
-    if a.dtype == BF16 and w.dtype == BF16 and k % 8 == 0 and lda % 8 == 0:
+    if a.dtype == BF16 and w.dtype == BF16 and _rows_aligned(a, k, lda):
         if not is_library_product(a, w):
             f = _fn("gemm_bf16", "kvf_gemm_bf16", _GEMM_BF16_ARGS)
             wp, tiled = _w_args(w)

@@ -394,6 +394,24 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
         assert all(torch.equal(x1, x2) for x1, x2 in zip(*got))
 
 
+@pytest.mark.parametrize("m", [5, 40])
+def test_gemm_rows_off_a_16_byte_boundary_take_the_plain_kernel(m):
+    """Rows that start two bytes past a 16-byte boundary cannot be read 16 bytes at a time: neither
+    the matrix-core kernel nor the library takes them, the fused forms refuse them, and the plain
+    kernel gives the product."""
+    g = torch.Generator().manual_seed(m)
+    wide = torch.randn(m, 104, generator=g).to(torch.bfloat16).to(DEV)
+    a = wide[:, 1:97]
+    w = (torch.randn(48, 96, generator=g) / 10).to(torch.bfloat16).to(DEV)
+    assert a.data_ptr() % 16 == 2 and a.stride(0) % 8 == 0
+    assert not ops().bf16_kernel_takes(a, w) and not ops().is_library_product(a, w)
+    out = torch.empty(m, 48, device=DEV)
+    ops().gemm(a, w, out)
+    torch.testing.assert_close(out.double().cpu(), a.double().cpu() @ w.double().cpu().T, atol=2e-5, rtol=2e-5)
+    with pytest.raises(ops().KernelError):
+        ops().gemm_fused(a, w, torch.empty(m, 24, dtype=torch.bfloat16, device=DEV), silu_pairs=True)
+
+
 def test_gemm_bf16_rows_do_not_depend_on_neighbours():
     g = torch.Generator().manual_seed(9)
     a = torch.randn(16, 2048, generator=g).to(torch.bfloat16).to(DEV)
