@@ -133,3 +133,29 @@ def test_refusals():
         fill_step(step, meta, [StepEntry("a", [1] * 65, 0)], cache.block_table, lambda r: -1, 4)
     with pytest.raises(ValueError):
         fill_step(step, meta, [], cache.block_table, lambda r: -1, 4)
+
+
+def test_workspace_hands_out_the_same_memory_until_it_grows():
+    """Scratch tensors are asked for by name, dtype and shape at every step: the same request gives
+    the same view, another shape of the same name shares its memory, and when a buffer has to
+    grow the views of the old one are not handed out again (graphs that were recorded with them
+    keep the old memory alive through ``snapshot``)."""
+    ws = Workspace("cpu")
+    a = ws.buf("x", (4, 8), torch.float32)
+    assert ws.buf("x", (4, 8), torch.float32) is a
+    b = ws.buf("x", (2, 8), torch.float32)
+    assert b.data_ptr() == a.data_ptr() and tuple(b.shape) == (2, 8)
+    other = ws.buf("x", (4, 8), torch.bfloat16)
+    assert other.data_ptr() != a.data_ptr()
+    kept = ws.snapshot()
+    big = ws.buf("x", (16, 8), torch.float32)
+    assert big.data_ptr() != a.data_ptr()
+    again = ws.buf("x", (4, 8), torch.float32)
+    assert again is not a and again.data_ptr() == big.data_ptr()
+    assert any(t.data_ptr() == a.data_ptr() for t in kept)
+    z = ws.zeros("flags", (8,), torch.int32)
+    assert int(z.sum()) == 0
+    ws.frozen = True
+    assert ws.buf("x", (4, 8), torch.float32) is again
+    with pytest.raises(RuntimeError, match="grow"):
+        ws.buf("x", (64, 8), torch.float32)
