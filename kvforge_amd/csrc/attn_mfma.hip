@@ -474,9 +474,15 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   const int j16 = lane % 16, kg = lane / 16;
   const int G = a.H / a.KV, D = a.d;
   const int chunks = (G + 15) / 16;
-  const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
+  // The kv heads are the fastest index of the grid: consecutive workgroups go to different
+  // XCDs, so the heads of one sequence pull on the cache through all of them, however its
+  // context compares with the others' (with the sequences in front, all workgroups of a sequence
+  // whose index is fixed modulo 8 landed on one XCD, and one long context among short ones was
+  // read through an eighth of the chip).
+  const int entry = blockIdx.y;
+  const int seq = seq_ids ? seq_ids[entry] : entry;
   if (seq < 0 || seq >= a.n_seqs) return;
-  const int kvh = blockIdx.y / chunks, tile = blockIdx.y - kvh * chunks;
+  const int kvh = blockIdx.x / chunks, tile = blockIdx.x - kvh * chunks;
   // without cu_q every sequence has one token, its own: nothing then waits for a load before the
   // query and the page lookups can be asked for
   const int q0 = cu_q ? cu_q[seq] : seq, qlen = cu_q ? cu_q[seq + 1] - q0 : 1, ctx = ctx_lens[seq];
@@ -601,7 +607,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   }
   if (!rows.ok[0]) return;
   const int head = rows.head[0];
-  const size_t slot = (static_cast<size_t>(blockIdx.x) * a.H + head) * a.splits + blockIdx.z;
+  const size_t slot = (static_cast<size_t>(entry) * a.H + head) * a.splits + blockIdx.z;
   if (a.splits > 1 && wave == 0 && kg == 0) {
     part_ml[slot * 2] = mm;  // in log2 units
     part_ml[slot * 2 + 1] = ll;
@@ -759,7 +765,8 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
     return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs)};
   const int G = H / KV, chunks = (G + 15) / 16;
-  const dim3 grid(num_seqs, KV * chunks, splits);
+  if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
+  const dim3 grid(KV * chunks, num_seqs, splits);
   switch (d / 16) {
 #define GO(DT)                                                                                      \
   case DT:                                                                                          \

@@ -20,6 +20,23 @@ ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup
 DECODE_KEYS_PER_SPLIT = 512
 MAX_DECODE_SPLITS = 64  # what the merge kernel takes (one lane per cut)
 COMPUTE_UNITS = 256
+DECODE_SKEW_MAX_CUTS = 8
+
+
+def skew_cuts(max_ctx: int, sum_ctx: int, n: int) -> int:
+    """Cuts of the key range that uneven contexts ask for, whatever the number of sequences: a
+    sequence's keys are walked by the waves of one workgroup per kv head and cut, so one long
+    context among short ones sets the step's time (measured at 32 sequences of 32 heads: 31
+    contexts of 600 and one of 32,768 take 153 us with one cut, 60 with eight; one of 8,192
+    takes 45 and 33).  The longest walk is brought down to about twice the mean one; a power of
+    two, so that captured launches change seldom."""
+    if n <= 1 or max_ctx < 4 * DECODE_KEYS_PER_SPLIT or sum_ctx <= 0:
+        return 1
+    want = min(max_ctx * n / (2.0 * sum_ctx), max_ctx // DECODE_KEYS_PER_SPLIT, DECODE_SKEW_MAX_CUTS)
+    cuts = 1
+    while cuts * 2 <= want:
+        cuts *= 2
+    return cuts
 
 
 @dataclass
@@ -162,6 +179,7 @@ class Step:
         self.host_token_ids: np.ndarray | None = None
         self.prefill_seqs: list[int] = []
         self.max_decode_ctx = 0
+        self.decode_skew = 1     # cuts of the key range asked for by uneven contexts (skew_cuts)
         self.max_position = 0
         self._work: dict[tuple[int, int], torch.Tensor | None] = {}
         self._identity_rotary = None
@@ -234,6 +252,8 @@ class Step:
         # Many sequences fill the chip by themselves.
         wgs = max(1, self.n_decode * KV * chunks)
         splits = max(1, min(COMPUTE_UNITS // wgs, ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS))
+        # uneven contexts: the longest one is cut further, however many sequences there are
+        splits = max(splits, min(self.decode_skew, max(1, ctx // DECODE_KEYS_PER_SPLIT)))
         if splits == 1:
             return 1, None
         acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)
@@ -395,6 +415,8 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
     step.host_token_ids = tok.copy()
     step.prefill_seqs = prefill
     step.max_decode_ctx = int(max((ctx[b] for b in decode), default=0))
+    live = [int(ctx[b]) for b in decode if ctx[b] > 0]
+    step.decode_skew = skew_cuts(step.max_decode_ctx, sum(live), len(live))
     step.max_position = int(ctx.max()) if Bp else 0
     step._work = {}
     return counts

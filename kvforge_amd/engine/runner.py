@@ -18,7 +18,7 @@ from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
 from kvforge_amd.engine.batch import (DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS, MetaBuffers, Step,
                                       StepEntry, Workspace, fill_step,
-                                      extend_tables)
+                                      extend_tables, skew_cuts)
 from kvforge_amd.kernels import ops
 from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
@@ -57,7 +57,7 @@ class ModelRunner:
         # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph;
         # only if every part's launches may be replayed for another batch
         self.use_graphs = bool(use_graphs) and all(p.replayable for p in model.spec.all_parts())
-        self.graphs: dict[tuple[int, int], _DecodeGraph] = {}
+        self.graphs: dict[tuple[int, tuple[int, int]], _DecodeGraph] = {}
         self.num_graph_replays = 0
         cap = self.meta.max_seqs
         # floats: temperatures, top-p, then MAX_DECODE_RUN rows of uniform numbers; ints: top-k,
@@ -214,6 +214,9 @@ class ModelRunner:
         # are kept per such cell, planned for the cell's lower edge.
         ctx_bucket = min(step.max_decode_ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
         step.max_decode_ctx = max(ctx_bucket * DECODE_KEYS_PER_SPLIT, 1)
+        # uneven contexts ask for further cuts (a power of two): a cell of its own
+        skew = skew_cuts(step.max_decode_ctx, sum(e.start_pos + 1 for e in entries), b)
+        step.decode_skew = skew
         cap = self.meta.max_seqs
         fh, ih = self._sample_f_np, self._sample_i_np
         ids = [e.request_id for e in entries]
@@ -237,7 +240,7 @@ class ModelRunner:
         if dirty:
             self._sample_f.copy_(self._sample_f_host, non_blocking=True)
         self._run_counter.zero_()
-        key = (bucket, ctx_bucket)
+        key = (bucket, (ctx_bucket, skew))
         graph = self.graphs.get(key)
         replays = k
         if graph is None:
@@ -265,7 +268,8 @@ class ModelRunner:
         if any(s + k > self.max_model_len for s in starts):
             return None
         ctx_bucket = min((max(starts) + 1) // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
-        graph = self.graphs.get((run.bucket, ctx_bucket))
+        skew = skew_cuts(max(ctx_bucket * DECODE_KEYS_PER_SPLIT, 1), sum(s + 1 for s in starts), len(starts))
+        graph = self.graphs.get((run.bucket, (ctx_bucket, skew)))
         if graph is None:
             return None
         base = k if run.base == 0 else 0

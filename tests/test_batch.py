@@ -159,3 +159,16 @@ def test_workspace_hands_out_the_same_memory_until_it_grows():
     assert ws.buf("x", (4, 8), torch.float32) is again
     with pytest.raises(RuntimeError, match="grow"):
         ws.buf("x", (64, 8), torch.float32)
+
+
+def test_uneven_contexts_ask_for_cuts_of_the_key_range():
+    from kvforge_amd.engine.batch import skew_cuts
+    assert skew_cuts(600, 32 * 600, 32) == 1                     # even contexts: none
+    assert skew_cuts(1800, 1800 + 31 * 100, 32) == 1             # too short to be worth a merge
+    assert skew_cuts(32768, 32768 + 31 * 600, 32) == 8           # one long context among short ones
+    assert skew_cuts(8192, 8192 + 31 * 600, 32) == 4
+    assert skew_cuts(8192, 8192 + 63 * 600, 64) == 4
+    assert skew_cuts(4352, 4352 + 31 * 300, 32) == 4
+    assert skew_cuts(3000, 3000 + 3000, 2) == 1                  # twice the mean is the aim
+    assert skew_cuts(2100, 2100 + 63 * 10, 64) == 4              # never cuts below 512 keys
+    assert skew_cuts(40000, 40000, 1) == 1                       # one sequence: the other rule's case

@@ -573,6 +573,34 @@ def test_graph_replay_of_library_products_at_the_served_width(tmp_path):
     assert again == graphed
 
 
+def test_one_long_context_among_short_ones(tmp_path):
+    """Twelve requests decode together, one of them past 2,300 tokens: the decode kernel then
+    cuts the key range although the sequences alone would fill the chip, in eager steps and in
+    captured ones (a cell of graphs of its own).  Every token is the plain model's choice within
+    bf16 rounding, for the long request and for short ones beside it."""
+    from tests.replay_util import TINY_C, sharpen
+    cfg = dict(TINY_C, max_position_embeddings=4096)
+    folder = str(tmp_path / "skew")
+    kvforge_amd.write_random_model(folder, cfg, seed=8)
+    sharpen(folder, 6.0)
+    oracle = Oracle(folder)
+    rng = random.Random(4)
+    prompts = [[rng.randrange(1, 200) for _ in range(2310)]] + prompts_for(200, 11, 9, 5, 40)
+    params = SamplingParams(max_tokens=18, temperature=0.0)
+    for use_graphs in (False, True):
+        config = EngineConfig(cache=CacheConfig(block_size=16, num_blocks=400),
+                              scheduler=SchedulerConfig(max_num_seqs=16, max_num_batched_tokens=1024,
+                                                        max_model_len=4096),
+                              dtype="bfloat16", use_graphs=use_graphs)
+        engine = InferenceEngine.from_folder(folder, config)
+        outs = [o.output_token_ids for o in engine.generate(prompts, params)]
+        if use_graphs:
+            assert any(skew > 1 for _, (_, skew) in engine.runner.graphs)
+        for i in (0, 1, 7):
+            oracle.check_choices(prompts[i], outs[i], 3e-2)
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
 def test_wide_layers_through_graphs_and_queued_runs(tmp_path):
     """A model whose layers are wide enough for the kernels a real model is served with (the down
     projection in two halves of K, one of them owed from layer to layer; two groups of columns
