@@ -4,16 +4,25 @@
 // Why this exists: a step that cannot be replayed from a graph (a portion of a prompt, whose
 // size changes from step to step) launches every kernel from the host, and four products per
 // layer through torch.mm cost 17 us of host time each, more than the device needs for them at a
-// few hundred rows.  Here a product's descriptors and the algorithm the library's heuristic
-// picks are made once per shape and kept; a call is then a table look-up and one
-// hipblasLtMatmul.
+// few hundred rows.  Here a product's descriptors and its algorithm are made once per shape and
+// kept; a call is then a table look-up and one hipblasLtMatmul.
+//
+// Which algorithm: the first the library's heuristic names, except for row counts that come
+// back all the time (the powers of two from 64 to 512: the padded batches of captured decode
+// steps).  For those the heuristic's first CANDIDATES answers are timed once,
+// on the operands of the first call that may be repeated (not an accumulating one, not under
+// stream capture) and with the caches swept before every run, and the fastest is kept: a decode
+// step of 64 sequences at the 1B shape goes from 1.72 to 1.54 ms.  The engine's first call
+// of a shape is such a call (captures follow an eager step), so a shape's algorithm is settled
+// before its first result is handed out and equal calls give equal bits within a process.
 //
 // hipBLASLt counts in column-major matrices.  Row-major C[M, N] is column-major C^T[N, M] =
 // op(W) * A^T: the first operand is W as a K x N column-major matrix (leading dimension K),
 // transposed; the second is A as K x M (leading dimension lda), as it is.
 //
 // The workspace is allocated once per device by kvf_gemm_library_init, which must be called
-// outside stream capture; the product itself allocates nothing and may be captured.
+// outside stream capture.  A product allocates nothing while its stream is being captured;
+// outside capture the first timing of candidates allocates the memory the caches are swept with.
 #include "common.h"
 
 #include <hipblaslt/hipblaslt.h>
@@ -24,11 +33,16 @@
 namespace {
 constexpr int MAX_DEVICES = 16;
 
+constexpr int CANDIDATES = 16;
+
 struct Plan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
-  hipblasLtMatmulAlgo_t algo;
+  hipblasLtMatmulAlgo_t algo;                  // the one in use
+  hipblasLtMatmulAlgo_t others[CANDIDATES];    // what the heuristic named, in its order
+  int num_others = 0;
   bool usable = false;
+  bool timed = true;                           // false: the candidates are still to be timed
 };
 
 struct Key {
@@ -45,10 +59,15 @@ struct KeyHash {
   }
 };
 
+// Memory that is overwritten between the timed runs of candidates, so that each run finds the
+// weights where a layer's first use finds them: in HBM, not in the 256 MB memory-side cache.
+constexpr size_t FLUSH_BYTES = 384u << 20;
+
 struct Device {
   hipblasLtHandle_t handle = nullptr;
   void* workspace = nullptr;
   size_t workspace_bytes = 0;
+  void* flush = nullptr;
   std::unordered_map<Key, Plan, KeyHash> plans;
 };
 Device g_dev[MAX_DEVICES];
@@ -70,17 +89,68 @@ Plan make_plan(Device& dv, const Key& k) {
   if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return p;
   const uint64_t room = dv.workspace_bytes;
   hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &room, sizeof(room));
-  hipblasLtMatmulHeuristicResult_t found[1];
+  // row counts that recur, up to where the heuristic's first answer is as good as any in place
+  // (at 2,048 rows the timed choice gained nothing in a whole prefill, at 64 it gains 11% of a
+  // decode step): their candidates are worth timing
+  const bool recurs = k.M >= 64 && k.M <= 512 && (k.M & (k.M - 1)) == 0;
+  hipblasLtMatmulHeuristicResult_t found[CANDIDATES];
   int count = 0;
-  const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(dv.handle, p.desc, p.w, p.a, p.c, p.c, pref, 1,
-                                                             found, &count);
+  const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(dv.handle, p.desc, p.w, p.a, p.c, p.c, pref,
+                                                             recurs ? CANDIDATES : 1, found, &count);
   hipblasLtMatmulPreferenceDestroy(pref);
-  if (st == HIPBLAS_STATUS_SUCCESS && count > 0 && found[0].state == HIPBLAS_STATUS_SUCCESS &&
-      found[0].workspaceSize <= dv.workspace_bytes) {
-    p.algo = found[0].algo;
+  if (st != HIPBLAS_STATUS_SUCCESS) return p;
+  for (int i = 0; i < count && i < CANDIDATES; ++i)
+    if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= dv.workspace_bytes)
+      p.others[p.num_others++] = found[i].algo;
+  if (p.num_others > 0) {
+    p.algo = p.others[0];
     p.usable = true;
+    p.timed = p.num_others < 2;
   }
   return p;
+}
+
+// Runs every candidate on the call's own operands (C is written with the same product each
+// time) and keeps the fastest: the best of TIMED_RUNS runs each, every run after the caches have
+// been swept, as a model's weights are cold when their layer comes round.  Waits for the stream:
+// only outside capture.
+constexpr int TIMED_RUNS = 4;
+
+void time_candidates(Device& dv, Plan& p, const void* A, const void* W, void* C, hipStream_t s) {
+  p.timed = true;
+  if (!dv.flush && hipMalloc(&dv.flush, FLUSH_BYTES) != hipSuccess) {
+    dv.flush = nullptr;
+    hipGetLastError();
+    return;  // no room to sweep the caches with: the heuristic's first answer stays
+  }
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    if (e0) hipEventDestroy(e0);
+    return;
+  }
+  const float alpha = 1.f, beta = 0.f;
+  float best = 0.f;
+  int best_i = -1;
+  for (int i = 0; i < p.num_others; ++i) {
+    float mine = 0.f;
+    bool ok = true;
+    for (int r = 0; r <= TIMED_RUNS && ok; ++r) {  // the first run is not counted
+      float ms = 0.f;
+      ok = hipMemsetAsync(dv.flush, r, FLUSH_BYTES, s) == hipSuccess && hipEventRecord(e0, s) == hipSuccess &&
+           hipblasLtMatmul(dv.handle, p.desc, &alpha, W, p.w, A, p.a, &beta, C, p.c, C, p.c, &p.others[i],
+                           dv.workspace, dv.workspace_bytes, s) == HIPBLAS_STATUS_SUCCESS &&
+           hipEventRecord(e1, s) == hipSuccess && hipEventSynchronize(e1) == hipSuccess &&
+           hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+      if (ok && r > 0 && (r == 1 || ms < mine)) mine = ms;
+    }
+    if (ok && (best_i < 0 || mine < best)) {
+      best = mine;
+      best_i = i;
+    }
+  }
+  if (best_i >= 0) p.algo = p.others[best_i];
+  hipEventDestroy(e0);
+  hipEventDestroy(e1);
 }
 }  // namespace
 
@@ -127,6 +197,11 @@ KVF_EXPORT int kvf_gemm_library_bf16(const void* A, const void* W, void* C, int 
     const Key key{M, N, K, lda, ldc, out_f32 ? 1 : 0};
     auto it = dv.plans.find(key);
     if (it == dv.plans.end()) it = dv.plans.emplace(key, make_plan(dv, key)).first;
+    if (it->second.usable && !it->second.timed && !accumulate) {
+      hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
+        time_candidates(dv, it->second, A, W, C, s);
+    }
     plan = it->second;
     ws = dv.workspace;
     ws_bytes = dv.workspace_bytes;
