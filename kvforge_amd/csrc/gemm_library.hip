@@ -8,7 +8,7 @@
 // kept; a call is then a table look-up and one hipblasLtMatmul.
 //
 // Which algorithm: the first the library's heuristic names, except for row counts that come
-// back all the time (the powers of two from 64 to 512: the padded batches of captured decode
+// back all the time (the powers of two from 32 to 512: the padded batches of captured decode
 // steps).  For those the heuristic's first CANDIDATES answers are timed once,
 // on the operands of the first call that may be repeated (not an accumulating one, not under
 // stream capture) and with the caches swept before every run, and the fastest is kept: a decode
@@ -92,7 +92,7 @@ Plan make_plan(Device& dv, const Key& k) {
   // row counts that recur, up to where the heuristic's first answer is as good as any in place
   // (at 2,048 rows the timed choice gained nothing in a whole prefill, at 64 it gains 11% of a
   // decode step): their candidates are worth timing
-  const bool recurs = k.M >= 64 && k.M <= 512 && (k.M & (k.M - 1)) == 0;
+  const bool recurs = k.M >= 32 && k.M <= 512 && (k.M & (k.M - 1)) == 0;
   hipblasLtMatmulHeuristicResult_t found[CANDIDATES];
   int count = 0;
   const hipblasStatus_t st = hipblasLtMatmulAlgoGetHeuristic(dv.handle, p.desc, p.w, p.a, p.c, p.c, pref,
