@@ -11,6 +11,10 @@
 // (three passes over the row each, weights summed per digit in LDS), which needs no sort and no
 // memory beyond the row itself.
 #include "common.h"
+#include "sampling_static.h"
+
+#include <cstdio>
+#include <mutex>
 
 namespace {
 constexpr int THREADS = 1024, NWAVES = THREADS / KVF_WAVE;
@@ -404,6 +408,76 @@ KVF_EXPORT int kvf_sample(const float* logits, int ld, int rows, int V, const fl
   if (rows <= 0) return 0;
   if (V <= 0 || ld < V || splits < 1 || splits > 64 || (splits > 1 && !work))
     return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(sample_kernel, dim3(rows, splits), dim3(THREADS), 0, s, logits, ld, V, temperature,
+                     top_k, top_p, u, u_step, u_stride, tokens, work);
+  return kvf_last_error();
+}
+
+namespace {
+// Work memory of kvf_sample_static: tickets, then the chunks' best values, then their indices.
+// The array is part of the library's image, so every GPU the library runs on holds a copy at an
+// address of its own.  In host code the name below only stands for the symbol; the device
+// address comes from hipGetSymbolAddress and is what launches are given.
+static __device__ __align__(256) int scratch[KVF_SAMPLE_STATIC_MAX_ROWS * (1 + 2 * KVF_SAMPLE_STATIC_MAX_SPLITS)];
+constexpr int MAX_DEVICES = 64;
+int* scratch_address[MAX_DEVICES];  // per device, looked up at the first call on it
+std::mutex scratch_lock;
+
+__global__ void clear_ints_kernel(int* __restrict__ p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// The device address of `scratch` on the current device; null (and *code set) if the runtime
+// does not give it.
+int* scratch_on_current_device(hipError_t* code) {
+  int dev = -1;
+  *code = hipGetDevice(&dev);
+  if (*code != hipSuccess) return nullptr;
+  if (dev < 0 || dev >= MAX_DEVICES) {
+    *code = hipErrorInvalidDevice;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (!scratch_address[dev]) {
+    void* p = nullptr;
+    *code = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (*code != hipSuccess || !p) {
+      if (*code == hipSuccess) *code = hipErrorInvalidSymbol;
+      return nullptr;
+    }
+    scratch_address[dev] = static_cast<int*>(p);
+  }
+  return scratch_address[dev];
+}
+}  // namespace
+
+KVF_EXPORT int kvf_sample_static(const float* logits, int ld, int rows, int V, const float* temperature,
+                                 const int* top_k, const float* top_p, const float* u,
+                                 const int* u_step, int u_stride, int* tokens, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (rows > KVF_SAMPLE_STATIC_MAX_ROWS) {
+    fprintf(stderr, "kvf_sample_static: %d rows asked for, at most %d fit its work memory\n", rows,
+            KVF_SAMPLE_STATIC_MAX_ROWS);
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (V <= 0 || ld < V) return static_cast<int>(hipErrorInvalidValue);
+  // about one workgroup per compute unit, each with at least 4096 logits
+  int splits = KVF_SAMPLE_STATIC_MAX_SPLITS;
+  if (splits > 256 / rows) splits = 256 / rows;
+  if (splits > V / 4096) splits = V / 4096;
+  if (splits < 1) splits = 1;
+  int* work = nullptr;
+  if (splits > 1) {
+    hipError_t code = hipSuccess;
+    work = scratch_on_current_device(&code);
+    if (!work) return static_cast<int>(code);
+    // the tickets start at zero whatever the call before left (a fill kernel, not a memset
+    // node: the launches may be captured)
+    hipLaunchKernelGGL(clear_ints_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, work, rows);
+    const int launched = kvf_last_error();
+    if (launched != 0) return launched;
+  }
   hipLaunchKernelGGL(sample_kernel, dim3(rows, splits), dim3(THREADS), 0, s, logits, ld, V, temperature,
                      top_k, top_p, u, u_step, u_stride, tokens, work);
   return kvf_last_error();

@@ -35,7 +35,7 @@ MODULE_FLAGS: dict[str, list[str]] = {"attn_mfma": ["-fno-honor-nans"]}
 # Libraries a module is linked against (after its sources on the command line).
 ROCM_LIB = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
 MODULE_LINK: dict[str, list[str]] = {"gemm_library": [f"-L{ROCM_LIB}", f"-Wl,-rpath,{ROCM_LIB}", "-lhipblaslt"]}
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "sampling_static.h"]
 MODULES: dict[str, list[str]] = {
     "elementwise": ["elementwise.hip"],
     "gemm_generic": ["gemm_generic.hip"],
