@@ -82,10 +82,10 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
                             temperature=0.0, ignore_eos=True)
     for p in random_prompts(vocab, batch, prompt_len, seed):
         engine.add_request(p, params)
-    while any(r.is_prefill for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
+    while any(not r.decoding for r in engine.scheduler.requests.values()) or engine.scheduler.num_waiting:
         engine.step()
-    run_limit = engine.config.decode_run_steps
-    run_ahead = engine.config.decode_run_ahead
+    sched = engine.scheduler
+    run_limit, run_ahead = sched.run_limit, sched.run_ahead
 
     def decode_steps(n):
         """Exactly ``n`` decode steps of the whole batch (the engine may take several between two
@@ -94,10 +94,10 @@ def decode_run(engine, vocab, batch, prompt_len, steps, warmup, seed=0):
         produced, start = 0, engine.runner.num_forward_passes
         while engine.runner.num_forward_passes - start < n:
             left = n - (engine.runner.num_forward_passes - start)
-            engine.config.decode_run_steps = min(run_limit, left)
-            engine.config.decode_run_ahead = run_ahead and left >= 2 * run_limit
+            sched.run_limit = min(run_limit, left)
+            sched.run_ahead = run_ahead and left >= 2 * run_limit
             produced += sum(len(o.new_token_ids) for o in engine.step())
-        engine.config.decode_run_steps, engine.config.decode_run_ahead = run_limit, run_ahead
+        sched.run_limit, sched.run_ahead = run_limit, run_ahead
         assert engine.runner.num_forward_passes - start == n
         return produced
 

@@ -145,12 +145,13 @@ class CacheManager:
         return max(0, need - have)
 
     # --------------------------------------------------------------- life cycle
-    def can_allocate(self, num_tokens: int) -> bool:
+    def can_allocate(self, num_tokens: int, reserve: bool = True) -> bool:
         """Room for a new request of ``num_tokens`` while keeping the watermark free
-        (src/tokenvault/cache/block_manager.py:165-170)."""
+        (src/tokenvault/cache/block_manager.py:165-170); ``reserve=False`` leaves the watermark
+        out, for a pool that is as empty as it will ever get."""
         if self.slots.num_slots and self.slots.num_free == 0:
             return False
-        return all(self._new_blocks(g, None, num_tokens) <= p.num_free - wm
+        return all(self._new_blocks(g, None, num_tokens) <= p.num_free - (wm if reserve else 0)
                    for g, (p, wm) in enumerate(zip(self.pools, self.watermark_blocks)))
 
     def allocate(self, request_id: str, num_tokens: int) -> None:

@@ -77,7 +77,7 @@ class ModelRunner:
         self._sample_f_host = torch.zeros(nf, dtype=torch.float32, pin_memory=True)
         self._sample_i_host = torch.zeros(cap, dtype=torch.int32, pin_memory=True)
         self._sample_f_np, self._sample_i_np = self._sample_f_host.numpy(), self._sample_i_host.numpy()
-        self._sample_ids: list[str] = []
+        self._sample_rows: list[tuple] = []
         self._sample_bucket = 0
         self._sample_drawn: list[int] = []
 
@@ -110,6 +110,10 @@ class ModelRunner:
         self.num_forward_passes += 1
         self.num_tokens_processed += step.n_tokens
         return logits
+
+    def takes_runs(self, num_requests: int) -> bool:
+        """Whether runs of decode steps on the device are possible for so many requests."""
+        return self.use_graphs and 0 < num_requests <= GRAPH_MAX_BATCH
 
     def graph_takes(self, entries: Sequence[StepEntry], num_params: int) -> bool:
         """Whether a step goes through the captured decode path: single tokens that each want
@@ -220,7 +224,11 @@ class ModelRunner:
         cap = self.meta.max_seqs
         fh, ih = self._sample_f_np, self._sample_i_np
         ids = [e.request_id for e in entries]
-        if ids != self._sample_ids or bucket != self._sample_bucket:
+        # who sits in which row, with what parameters: an id that was freed and is used again
+        # (another serial) or comes with other parameters is another occupant
+        rows = [(e.request_id, self.cache.serial(e.request_id), p.temperature, p.top_p, p.top_k)
+                for e, p in zip(entries, params)]
+        if rows != self._sample_rows or bucket != self._sample_bucket:
             # the batch changed: rewrite the per-row parameters (padding rows are greedy)
             fh[:bucket] = 0.0
             fh[cap:cap + bucket] = 1.0
@@ -228,7 +236,7 @@ class ModelRunner:
             ih[:bucket] = 0
             for i, p in enumerate(params):
                 fh[i], fh[cap + i], ih[i] = p.temperature, p.top_p, p.top_k
-            self._sample_ids, self._sample_bucket = ids, bucket
+            self._sample_rows, self._sample_bucket = rows, bucket
             self._sample_drawn = [i for i, p in enumerate(params) if not p.greedy]
             self._sample_i[:cap].copy_(self._sample_i_host, non_blocking=True)
             dirty = True

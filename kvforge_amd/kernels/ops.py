@@ -62,6 +62,17 @@ def _check(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True) 
         raise KernelError(f"{name} must be contiguous")
 
 
+def _overlap(a: torch.Tensor, b: torch.Tensor) -> bool:
+    """Whether the memory spanned by two tensors' storage views intersects."""
+    def span(t):
+        if t.numel() == 0:
+            return t.data_ptr(), t.data_ptr()
+        last = sum((n - 1) * st for n, st in zip(t.shape, t.stride()))
+        return t.data_ptr(), t.data_ptr() + (last + 1) * t.element_size()
+    (a0, a1), (b0, b1) = span(a), span(b)
+    return a0 < b1 and b0 < a1
+
+
 def _ok(code: int, what: str) -> None:
     if code != 0:
         raise KernelError(f"{what} failed with HIP error {code}")
@@ -252,6 +263,13 @@ def plain_of(w) -> torch.Tensor:
     return w.plain if isinstance(w, StreamedWeight) else w
 
 
+def copies_of(w) -> list[torch.Tensor]:
+    """Every tensor that holds ``w``: the matrix itself, and its tiles if it is streamed."""
+    if isinstance(w, StreamedWeight):
+        return [w.plain, w.tiles]
+    return [] if w is None else [w]
+
+
 def _w_args(w) -> tuple[int, int]:
     """(pointer, tiled flag) of a weight for the weight-streaming kernel."""
     if isinstance(w, StreamedWeight):
@@ -377,6 +395,11 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
             raise KernelError(f"gemm: {name} must have the row stride of out")
     if half_out is not None and not k_halves_pay(a, w):
         raise KernelError("gemm: half_out only where k_halves_pay(a, w)")
+    if half_out is not None:
+        # the workgroups of one half of K read owed and out while those of the other write half_out
+        for t, name in ((owed, "owed"), (out, "out")):
+            if t is not None and _overlap(t, half_out):
+                raise KernelError(f"gemm: half_out must not share memory with {name}")
     if m == 0:
         return
     out_kind = 2 if accumulate else (0 if out.dtype == F32 else 1)

@@ -94,6 +94,16 @@ class Transformer:
         total = sum(p.num_bytes() for p in (spec.embedding, spec.final_norm, spec.head, *spec.positions))
         return total + sum(spec.blocks[c.layer].num_bytes() for c in self.order)
 
+    @property
+    def resident_bytes(self) -> int:
+        """Bytes the weights occupy on the device, every copy and layout counted (a tensor that
+        two parts share counts once)."""
+        seen: dict[int, int] = {}
+        for p in self.spec.all_parts():
+            for t in p.held_tensors():
+                seen[t.data_ptr()] = t.numel() * t.element_size()
+        return sum(seen.values())
+
     # ------------------------------------------------------------------ forward
     def forward(self, step) -> torch.Tensor:
         """Runs the step's tokens from the cache; returns fp32 logits ``[n_logits, vocab]`` (a

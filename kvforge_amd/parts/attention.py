@@ -93,6 +93,9 @@ class PagedAttention(Mixer):
         return sum(t.numel() * t.element_size()
                    for t in map(ops.plain_of, (self.w_qkv, self.w_o)) if t is not None)
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        return ops.copies_of(self.w_qkv) + ops.copies_of(self.w_o)
+
     def seal(self) -> None:
         self.w_qkv, self.w_o = ops.streamed(ops.plain_of(self.w_qkv)), ops.streamed(ops.plain_of(self.w_o))
 

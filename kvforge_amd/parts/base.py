@@ -88,6 +88,11 @@ class Part:
         """Bytes of weights this part reads in one step."""
         return 0
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        """The device tensors this part keeps for its weights, every copy and layout of them
+        (what the weights occupy, as opposed to what a step reads)."""
+        return []
+
     def seal(self) -> None:
         """Called once after ``load`` (and any ``absorb_norm``), before the first forward: the
         place for the last re-layout of weights, such as tiles for the weight-streaming kernel."""
@@ -182,6 +187,9 @@ class Block(Part):
     def num_bytes(self) -> int:
         return sum(p.num_bytes() for p in self.parts())
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        return [t for p in self.parts() for t in p.held_tensors()]
+
     @property
     def replayable(self) -> bool:
         return all(p.replayable for p in self.parts())
@@ -207,6 +215,11 @@ def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.
         step.owe(residual, product)
     elif ops.k_halves_pay(a, w) and residual.is_contiguous():
         half = step.ws.buf("owed_half", tuple(residual.shape), torch.float32)
+        if owed is not None and owed.data_ptr() == half.data_ptr():
+            # what the caller took from the step is the half the product before this one left
+            # there: this product's workgroups read it while others write their half, so the
+            # new half goes to the other of two buffers
+            half = step.ws.buf("owed_half_other", tuple(residual.shape), torch.float32)
         ops.gemm(a, w, residual, accumulate=True, owed=owed, half_out=half)
         step.owe(residual, half)
     else:

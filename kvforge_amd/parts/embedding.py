@@ -26,6 +26,9 @@ class TokenEmbedding(Part):
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"elementwise"}
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        return [] if self.table is None else [self.table]
+
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed(ids, self.table, out)
 
@@ -54,6 +57,9 @@ class LMHead(Part):
     def num_bytes(self) -> int:
         w = ops.plain_of(self.weight)
         return w.numel() * w.element_size() if w is not None else 0
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return ops.copies_of(self.weight)
 
     def seal(self) -> None:
         # a tied table stays as it is for the embedding; the head streams a tiled copy

@@ -54,6 +54,9 @@ class SwiGLU(FeedForward):
         return sum(t.numel() * t.element_size()
                    for t in map(ops.plain_of, (self.w_gate_up, self.w_down)) if t is not None)
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        return ops.copies_of(self.w_gate_up) + ops.copies_of(self.w_down)
+
     def seal(self) -> None:
         self.w_gate_up = ops.streamed(ops.plain_of(self.w_gate_up))
         self.w_down = ops.streamed(ops.plain_of(self.w_down))

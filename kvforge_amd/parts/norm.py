@@ -31,6 +31,9 @@ class RMSNorm(Norm):
     def num_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
 
+    def held_tensors(self) -> list[torch.Tensor]:
+        return [] if self.weight is None else [self.weight]
+
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None,
                 add: torch.Tensor | None = None) -> None:
         ops.rmsnorm(x, self.weight, self.eps, out, rows, add)

@@ -17,8 +17,17 @@ import json
 import os
 import sys
 
-BLOCK_SIZE = 16
-MAX_LIVE = 16
+
+
+def pool_pages(max_tokens: int, block_size: int) -> int:
+    """Pages for ``max_tokens`` tokens of live requests, each request's count rounded up to a
+    multiple of 64 by the caller: a unit of 64 tokens takes ``ceil(64 / block_size)`` pages (a
+    request's pages are its own, so a page size that does not divide 64 rounds every unit up);
+    pages larger than 64 tokens round the total up to their own size."""
+    if block_size >= 64:
+        return max(1, -(-max_tokens // block_size))
+    units = max(1, -(-max_tokens // 64))
+    return units * -(-64 // block_size)
 
 
 def _say(msg: str) -> None:
@@ -33,7 +42,11 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--out", required=True, help="folder the logits files are written to")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--max-live", type=int, default=16, help="most requests live at a time")
     args = ap.parse_args(argv)
+    if args.block_size < 1 or args.max_live < 1 or args.max_tokens < 1:
+        ap.error("--block-size, --max-live and --max-tokens must be positive")
 
     _say("loading torch ...")
     import numpy as np
@@ -51,11 +64,12 @@ def main(argv: list[str] | None = None) -> int:
     dtype = parse_dtype(args.dtype)
     _say(f"loading model from {args.model} as {args.dtype}")
     model = Transformer.from_folder(args.model, dtype, "cuda")
-    capacity = max(64, -(-args.max_tokens // 64) * 64)
-    num_blocks = capacity // BLOCK_SIZE
-    runner = ModelRunner(model, BLOCK_SIZE, num_blocks, max_num_seqs=MAX_LIVE,
+    block_size = args.block_size
+    num_blocks = pool_pages(args.max_tokens, block_size)
+    capacity = num_blocks * block_size
+    runner = ModelRunner(model, block_size, num_blocks, max_num_seqs=args.max_live,
                          max_num_batched_tokens=capacity, max_model_len=capacity)
-    _say(f"ready: {num_blocks} pages of {BLOCK_SIZE} tokens per cache group")
+    _say(f"ready: {num_blocks} pages of {block_size} tokens per cache group")
     held: dict[str, int] = {}
     cache = runner.cache
     while True:
@@ -71,7 +85,7 @@ def main(argv: list[str] | None = None) -> int:
         for e in rec.get("entries", []):
             rid, toks = str(e["id"]), [int(t) for t in e["tokens"]]
             if not toks:
-                continue
+                raise ValueError(f"step {sid}: request {rid} brings no tokens")
             start = held.get(rid, 0)
             if rid not in held:
                 cache.allocate(rid, 0)

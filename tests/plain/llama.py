@@ -33,11 +33,30 @@ def read_config(folder: str) -> dict[str, Any]:
 
 
 # --------------------------------------------------------------------------- parts
+def _wide(x: torch.Tensor) -> torch.Tensor:
+    """``x.float()`` as the reference writes it; a float64 tensor stays float64, so that the same
+    functions also give a reference that is all but free of rounding (``forward(..., dtype=
+    torch.float64)``), against which the rounding of a 32-bit implementation can be measured."""
+    return x if x.dtype == torch.float64 else x.float()
+
+
+def _stored(x: torch.Tensor, store: torch.dtype | None) -> torch.Tensor:
+    """What a tensor is after the reference has stored it in its model dtype ``store`` (rounded
+    to bfloat16 and widened again), or unchanged for ``None``.  With ``store=torch.bfloat16``
+    ``forward`` reproduces the arithmetic of the reference run with ``dtype=bfloat16``
+    (src/tokenvault/config.py:143,150-151): every tensor between two operations, the residual
+    stream included, holds bfloat16 values, while norms, rotation, scores and softmax are
+    computed in 32-bit and rounded once (src/tokenvault/model.py:36-38,61;
+    src/tokenvault/cache/paged_attention.py:85-89)."""
+    return x if store is None else x.to(store).to(x.dtype)
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """src/tokenvault/model.py:35-38 — eps inside the rsqrt, weight multiplied in fp32."""
-    xf = x.float()
+    """src/tokenvault/model.py:35-38 — eps inside the rsqrt, weight multiplied in fp32 (in the
+    precision of ``x`` when that is float64)."""
+    xf = _wide(x)
     xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
-    return xf * weight.float()
+    return xf * weight.to(xf.dtype)
 
 
 def rope_inv_freq(head_dim: int, theta: float) -> torch.Tensor:
@@ -82,7 +101,8 @@ def rotate_half(x: torch.Tensor) -> torch.Tensor:
 def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """src/tokenvault/model.py:58-61 — ``x: [T, heads, d]``, ``cos/sin: [T, d]``."""
     cos, sin = cos.unsqueeze(-2), sin.unsqueeze(-2)
-    return x.float() * cos + rotate_half(x.float()) * sin
+    x = _wide(x)
+    return x * cos.to(x.dtype) + rotate_half(x) * sin.to(x.dtype)
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
@@ -94,36 +114,40 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: f
     group = q.shape[1] // k.shape[1]
     kk = k.repeat_interleave(group, dim=1)
     vv = v.repeat_interleave(group, dim=1)
-    scores = torch.einsum("qhd,lhd->hql", q.float(), kk.float()) * scale
+    scores = torch.einsum("qhd,lhd->hql", _wide(q), _wide(kk)) * scale
     q_pos = torch.arange(q.shape[0])[:, None] + q_offset
     k_pos = torch.arange(k.shape[0])[None, :]
     visible = k_pos <= q_pos
     if window is not None:
         visible = visible & (k_pos > q_pos - window)
     scores = scores.masked_fill(~visible[None], float("-inf"))
-    return torch.einsum("hql,lhd->qhd", torch.softmax(scores, -1), vv.float())
+    return torch.einsum("hql,lhd->qhd", torch.softmax(scores, -1), _wide(vv))
 
 
 def swiglu(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor,
-           down_w: torch.Tensor) -> torch.Tensor:
+           down_w: torch.Tensor, store: torch.dtype | None = None,
+           out_store: torch.dtype | None = None) -> torch.Tensor:
     """src/tokenvault/model.py:131-132 — ``down(silu(gate(x)) * up(x))``, weights ``[out, in]``."""
-    g = x @ gate_w.float().T
-    u = x @ up_w.float().T
-    return (torch.nn.functional.silu(g) * u) @ down_w.float().T
+    g = _stored(x @ gate_w.to(x.dtype).T, store)
+    u = _stored(x @ up_w.to(x.dtype).T, store)
+    act = _stored(_stored(torch.nn.functional.silu(g), store) * u, store)
+    return _stored(act @ down_w.to(x.dtype).T, out_store)
 
 
 def attention_block(x: torch.Tensor, w: dict[str, torch.Tensor], prefix: str, cfg: dict,
-                    cos: torch.Tensor, sin: torch.Tensor, window: int | None) -> torch.Tensor:
+                    cos: torch.Tensor, sin: torch.Tensor, window: int | None,
+                    store: torch.dtype | None = None,
+                    out_store: torch.dtype | None = None) -> torch.Tensor:
     """src/tokenvault/model.py:77-92 without the cache: project, rotate q and k, attend,
     project out."""
     T = x.shape[0]
     H, KV, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
-    q = (x @ w[prefix + "q_proj.weight"].float().T).view(T, H, d)
-    k = (x @ w[prefix + "k_proj.weight"].float().T).view(T, KV, d)
-    v = (x @ w[prefix + "v_proj.weight"].float().T).view(T, KV, d)
-    q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
-    out = causal_attention(q, k, v, 1.0 / math.sqrt(d), 0, window)
-    return out.reshape(T, H * d) @ w[prefix + "o_proj.weight"].float().T
+    q = _stored(x @ w[prefix + "q_proj.weight"].to(x.dtype).T, store).view(T, H, d)
+    k = _stored(x @ w[prefix + "k_proj.weight"].to(x.dtype).T, store).view(T, KV, d)
+    v = _stored(x @ w[prefix + "v_proj.weight"].to(x.dtype).T, store).view(T, KV, d)
+    q, k = _stored(apply_rope(q, cos, sin), store), _stored(apply_rope(k, cos, sin), store)
+    out = _stored(causal_attention(q, k, v, 1.0 / math.sqrt(d), 0, window), store)
+    return _stored(out.reshape(T, H * d) @ w[prefix + "o_proj.weight"].to(x.dtype).T, out_store)
 
 
 def inv_freq_for(cfg: dict) -> torch.Tensor:
@@ -143,24 +167,38 @@ def layer_window(cfg: dict, i: int) -> int | None:
 
 
 def forward(w: dict[str, torch.Tensor], cfg: dict, token_ids: list[int],
-            first_position: int = 0) -> torch.Tensor:
+            first_position: int = 0, dtype: torch.dtype = torch.float32,
+            residual_in_fp32: bool = False) -> torch.Tensor:
     """src/tokenvault/model.py:175-191 for one whole sequence: logits ``[T, vocab]`` in fp32.
-    ``first_position`` shifts every position (only distances count under rotary)."""
+    ``first_position`` shifts every position (only distances count under rotary).
+    ``dtype=torch.float64`` computes everything but the rotary angles (which are 32-bit by
+    definition) in double precision.  ``dtype=torch.bfloat16`` gives what the reference computes
+    when it runs in bfloat16 (see ``_stored``), returned in fp32 like its logits
+    (src/tokenvault/batching/continuous.py:117).  With ``residual_in_fp32`` only the tensors
+    *between* operations are rounded (normalised rows, q, k, v, attention output, the gated
+    feed-forward activation, the final normalised rows), while the residual stream, the products
+    added to it and the logits stay 32-bit: the least rounding a bfloat16 engine with a 32-bit
+    residual sum can do."""
+    store = stream = None
+    if dtype == torch.bfloat16:
+        store, dtype = torch.bfloat16, torch.float32
+        stream = None if residual_in_fp32 else store
     ids = torch.tensor(token_ids, dtype=torch.long)
-    h = w["model.embed_tokens.weight"].float()[ids]                      # model.py:169-170
+    h = w["model.embed_tokens.weight"][ids].to(dtype)                    # model.py:169-170
     pos = torch.arange(len(token_ids)) + first_position
     cos, sin = rope_cos_sin(pos, inv_freq_for(cfg))
     eps = cfg["rms_norm_eps"]
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
-        a = rms_norm(h, w[p + "input_layernorm.weight"], eps)
-        h = h + attention_block(a, w, p + "self_attn.", cfg, cos, sin, layer_window(cfg, i))
-        m = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
-        h = h + swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                       w[p + "mlp.down_proj.weight"])                     # model.py:186-187
-    hidden = rms_norm(h, w["model.norm.weight"], eps)                    # model.py:188
+        a = _stored(rms_norm(h, w[p + "input_layernorm.weight"], eps), store)
+        h = _stored(h + attention_block(a, w, p + "self_attn.", cfg, cos, sin,
+                                        layer_window(cfg, i), store, stream), stream)
+        m = _stored(rms_norm(h, w[p + "post_attention_layernorm.weight"], eps), store)
+        h = _stored(h + swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                               w[p + "mlp.down_proj.weight"], store, stream), stream)   # model.py:186-187
+    hidden = _stored(rms_norm(h, w["model.norm.weight"], eps), store)    # model.py:188
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
-    return hidden @ head.float().T                                       # model.py:157-158,190-191
+    return _stored(hidden @ head.to(hidden.dtype).T, stream)            # model.py:157-158,190-191
 
 
 def greedy(w: dict[str, torch.Tensor], cfg: dict, prompt: list[int], n: int) -> list[int]:

@@ -61,9 +61,26 @@ def assert_greedy_equal(got, want, gaps, margin=1e-4):
 
 
 @pytest.fixture(scope="module")
+def model_a_flat(tmp_path_factory):
+    """Tiny A exactly as the baseline configuration words it: N(0, 0.02) weights, tied head.
+    Its greedy output repeats the prompt's last token whatever the context, so only the test of
+    that configuration uses it."""
+    folder = str(tmp_path_factory.mktemp("tiny_a_flat"))
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-a"), seed=0)
+    return folder, Oracle(folder)
+
+
+@pytest.fixture(scope="module")
 def model_a(tmp_path_factory):
+    """Tiny A with peaked attention and layer outputs that outweigh the embedding: its next
+    token depends on what the cache holds (checked here for the kinds of prompt the tests use),
+    so a test of generated tokens fails on a broken cache."""
+    from tests.replay_util import context_matters, liven
     folder = str(tmp_path_factory.mktemp("tiny_a"))
     kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-a"), seed=0)
+    liven(folder)
+    assert context_matters(folder, prompts_for(256, 6, 2) + prompts_for(256, 4, 1)
+                           + [list(range(1, 60)), list(range(100, 140)), [7, 7, 7], [5, 17, 3]])
     return folder, Oracle(folder)
 
 
@@ -88,9 +105,9 @@ def prompts_for(vocab, n, seed, lo=2, hi=30):
     return [[rng.randrange(1, vocab) for _ in range(rng.randint(lo, hi))] for _ in range(n)]
 
 
-def test_baseline_config_a(model_a):
+def test_baseline_config_a(model_a_flat):
     """Tiny Llama A, fp32, seed 0, block 16: prompts of 5/17/33 tokens, greedy, 16 new each."""
-    folder, oracle = model_a
+    folder, oracle = model_a_flat
     g = torch.Generator().manual_seed(0)
     prompts = [torch.randint(0, 256, (n,), generator=g).tolist() for n in (5, 17, 33)]
     engine = engine_for(folder, block_size=16, num_blocks=64)
@@ -131,8 +148,8 @@ def test_batched_output_equals_isolated_greedy(model_a, dtype):
         assert len(o.output_token_ids) == 10
         if dtype == "float32":
             want, gaps = oracle.greedy(p, 10)
-            assert min(gaps) > 1e-4
-            assert o.output_token_ids == want
+            assert_greedy_equal(o.output_token_ids, want, gaps)
+            oracle.check_choices(p, o.output_token_ids, 1e-4)
         else:
             oracle.check_choices(p, o.output_token_ids, 3e-2)
 
@@ -185,6 +202,33 @@ def test_pages_run_out_preemption_preserves_outputs(model_a):
     for p, o in zip(prompts, outs):
         want, gaps = oracle.greedy(p, 10)
         assert_greedy_equal(o.output_token_ids, want, gaps)
+        oracle.check_choices(p, o.output_token_ids, 1e-4)
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
+def test_a_preempted_request_is_fed_again_into_pages_others_have_used(model_a):
+    """Two requests outgrow a pool of six pages: the later one loses its pages in the middle of
+    decoding, the earlier one grows into them, and the later one comes back under its own id,
+    is fed prompt and generated tokens again into pages that held the other's keys, and goes
+    on.  Every token of both is the plain model's choice."""
+    folder, oracle = model_a
+    prompts = [[9, 200, 31, 77, 5, 150, 42], [120, 8, 66, 201, 13, 90, 3]]
+    params = SamplingParams(max_tokens=12, temperature=0.0)
+    engine = engine_for(folder, block_size=4, num_blocks=6, max_num_seqs=2, decode_run_steps=1)
+    ids = [engine.add_request(p, params) for p in prompts]
+    second = engine.scheduler.requests[ids[1]]
+    outs, seen_back = {}, False
+    while engine.has_unfinished_requests():
+        for o in engine.step():
+            outs[o.request_id] = o
+        if second.num_preemptions and second.status == RequestStatus.RUNNING and not second.is_finished:
+            seen_back = True
+    assert second.num_preemptions >= 1 and seen_back
+    for rid, p in zip(ids, prompts):
+        assert len(outs[rid].output_token_ids) == 12
+        oracle.check_choices(p, outs[rid].output_token_ids, 1e-4)
+        want, gaps = oracle.greedy(p, 12)
+        assert_greedy_equal(outs[rid].output_token_ids, want, gaps)
     assert engine.cache.num_free_blocks == engine.cache.num_blocks
 
 
@@ -207,21 +251,25 @@ def test_abort_mid_generation(model_a):
     engine.step()
     engine.step()
     req = engine.scheduler.requests[rid]
-    assert req.status == RequestStatus.RUNNING
+    assert req.status == RequestStatus.RUNNING and req.num_output_tokens >= 2
     assert engine.abort_request(rid)
     assert req.status == RequestStatus.ABORTED and not engine.has_unfinished_requests()
+    assert engine.stats()["metrics"]["requests_aborted"] == 1
     assert engine.cache.num_free_blocks == engine.cache.num_blocks
     assert not engine.abort_request(rid)
 
 
 def test_stop_token_and_metrics(model_a):
     folder, oracle = model_a
-    want, _ = oracle.greedy([7, 7, 7], 10)
-    stop = want[3]
+    want, gaps = oracle.greedy([7, 7, 7], 10)
+    # a token that first appears some way into the output, so that stopping there is an event
+    at = next(i for i in range(2, 10) if want[i] not in want[:i])
+    assert min(gaps[:at + 1]) > 1e-4
+    stop = want[at]
     engine = engine_for(folder)
     out = engine.generate([[7, 7, 7]], SamplingParams(max_tokens=10, temperature=0,
                                                       stop_token_ids=[stop]))[0]
-    assert out.output_token_ids == want[: want.index(stop) + 1]
+    assert out.output_token_ids == want[:at + 1] and len(out.output_token_ids) >= 3
     assert out.finish_reason.value == "stop"
     stats = engine.stats()
     m = stats["metrics"]
@@ -235,6 +283,7 @@ def test_stop_token_and_metrics(model_a):
     untied = sum(t.numel() * 4 for n, t in tensors.items() if n.endswith("embed_tokens.weight")
                  and "lm_head.weight" in tensors)
     assert stats["weights_bytes"] == every - untied
+    assert stats["weights_bytes_resident"] == every       # fp32: one copy of every tensor
 
 
 def test_sampling_does_not_depend_on_batching(model_b):
@@ -424,7 +473,7 @@ def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
     preempted; some carry stop tokens, two are aborted.  In fp32 a token does not depend on its
     batch, so every way of running (single steps, runs, runs queued ahead) must give every
     request the same tokens and the same end, and give every page back."""
-    folder, _ = model_a
+    folder, oracle = model_a
     rng = random.Random(seed)
     n = 12
     prompts = prompts_for(256, n, 100 + seed, 1, 30)
@@ -436,7 +485,7 @@ def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
     aborted = {rng.randrange(n): rng.randint(3, 30), rng.randrange(n): rng.randint(3, 30)}
 
     def run(**kw):
-        engine = engine_for(folder, "float32", block_size=4, num_blocks=40, max_num_seqs=6,
+        engine = engine_for(folder, "float32", block_size=4, num_blocks=26, max_num_seqs=6,
                             max_num_batched_tokens=32, seed=5, **kw)
         ids, outs, step = {}, {}, 0
         while len(ids) < n or engine.has_unfinished_requests():
@@ -456,6 +505,18 @@ def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
 
     want, single = run(decode_run_steps=1)
     assert len(want) >= n - 2
+    # the single-step run is held to the plain model: greedy requests by their choices, drawn
+    # ones by the plain sampling rule on the plain logits of their own history
+    for i, (tokens, _) in want.items():
+        if params[i].greedy:
+            oracle.check_choices(prompts[i], tokens, 1e-4)
+        else:
+            logits = oracle.logits(prompts[i] + tokens)
+            for j, tok in enumerate(tokens):
+                probs = plain_sampling.processed_probs(logits[len(prompts[i]) - 1 + j],
+                                                       params[i].temperature, params[i].top_k)
+                u = plain_sampling.uniform(5, 7, j)
+                assert plain_sampling.draw_margin(probs, u, tok) < 1e-4, (i, j, tok)
     saw_ahead = 0
     for kw in (dict(decode_run_steps=8, decode_run_ahead=False), dict(decode_run_steps=8, decode_run_ahead=True),
                dict(decode_run_steps=3, decode_run_ahead=True)):
@@ -464,6 +525,92 @@ def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
         saw_ahead += engine.runner.num_runs_read_ahead
     assert single.scheduler.num_preemptions > 0 or seed != 0   # the pool is meant to run out
     assert saw_ahead > 0                                        # and runs are meant to be queued ahead
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_an_id_used_again_brings_its_own_sampling_parameters(model_b, use_graphs):
+    """Request "a" runs greedy to its end; then "a" again, alone, with a temperature, then once
+    more greedy.  Each must be what a fresh engine gives for those parameters: the rows of
+    sampling parameters that the captured decode path keeps on the device are keyed by who sits
+    in them, not by the id's string."""
+    folder, oracle = model_b
+    prompt = [3, 14, 15, 92, 65, 35]
+    greedy = SamplingParams(max_tokens=9, temperature=0.0)
+    drawn = SamplingParams(max_tokens=9, temperature=0.8, seed=11)
+
+    def run_a(engine, params):
+        engine.add_request(prompt, params, request_id="a")
+        final = None
+        while engine.has_unfinished_requests():
+            for o in engine.step():
+                final = o
+        assert final.request_id == "a" and final.finished
+        return final.output_token_ids
+
+    def fresh():
+        return engine_for(folder, block_size=8, seed=4, use_graphs=use_graphs)
+
+    want_greedy, want_drawn = run_a(fresh(), greedy), run_a(fresh(), drawn)
+    assert want_greedy != want_drawn
+    oracle.check_choices(prompt, want_greedy, 1e-4)
+    engine = fresh()
+    for params, want in ((greedy, want_greedy), (drawn, want_drawn), (greedy, want_greedy),
+                         (drawn, want_drawn)):
+        assert run_a(engine, params) == want, params
+
+
+@pytest.mark.parametrize("run", [1, 8])
+def test_the_models_length_ends_a_request_inside_a_run(model_b, run):
+    """``max_model_len`` 40: a request of 29 prompt tokens that asks for 50 more ends with
+    ``length`` after the 11th, whether the device takes its decode steps one by one or in runs
+    (the last run is cut to the room that is left)."""
+    folder, oracle = model_b
+    prompt = prompts_for(384, 1, 77, 29, 29)[0]
+    cfg = EngineConfig(cache=CacheConfig(block_size=8, num_blocks=32),
+                       scheduler=SchedulerConfig(max_num_seqs=4, max_num_batched_tokens=64, max_model_len=40),
+                       dtype="float32", decode_run_steps=run)
+    engine = InferenceEngine.from_folder(folder, cfg)
+    out = engine.generate([prompt], SamplingParams(max_tokens=50, temperature=0.0))[0]
+    assert out.finish_reason.value == "length" and len(prompt) + len(out.output_token_ids) == 40
+    oracle.check_choices(prompt, out.output_token_ids, 1e-4)
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+    if run > 1:
+        assert engine.runner.num_graph_replays > 0
+
+
+def test_more_requests_than_the_captured_decode_path_takes(model_b):
+    """140 requests decode together: beyond the largest captured batch (128) every step is
+    launched kernel by kernel; as requests end the batch falls below it and the captured path
+    takes over.  All tokens are the plain model's choices within bf16 rounding."""
+    from kvforge_amd.engine.runner import GRAPH_MAX_BATCH
+    folder, oracle = model_b
+    n = GRAPH_MAX_BATCH + 12
+    prompts = prompts_for(384, n, 31, 2, 12)
+    params = [SamplingParams(max_tokens=4 + (i % 9), temperature=0.0) for i in range(n)]
+    cfg = EngineConfig(cache=CacheConfig(block_size=8, num_blocks=1024),
+                       scheduler=SchedulerConfig(max_num_seqs=n, max_num_batched_tokens=2048),
+                       dtype="bfloat16")
+    engine = InferenceEngine.from_folder(folder, cfg)
+    outs = engine.generate(prompts, params)
+    assert max(engine.metrics.batch_sizes) == n and engine.runner.num_graph_replays > 0
+    assert [len(o.output_token_ids) for o in outs] == [p.max_tokens for p in params]
+    for i in range(0, n, 7):
+        oracle.check_choices(prompts[i], outs[i].output_token_ids, 3e-2)
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
+def test_a_model_stored_in_two_files_generates_the_same_tokens(model_b, tmp_path):
+    import shutil
+    from kvforge_amd.weights import write_safetensors
+    folder, oracle = model_b
+    sharded = str(tmp_path / "sharded")
+    shutil.copytree(folder, sharded)
+    write_safetensors(sharded, kvforge_amd.read_safetensors_folder(folder), shards=2)
+    prompts = prompts_for(384, 3, 5, 4, 30)
+    want = [o.output_token_ids for o in engine_for(folder, block_size=8).generate(prompts, GREEDY)]
+    got = [o.output_token_ids for o in engine_for(sharded, block_size=8).generate(prompts, GREEDY)]
+    assert got == want
+    oracle.check_choices(prompts[2], got[2], 1e-4)
 
 
 def test_rejections_at_the_entry_point(model_a):
@@ -506,6 +653,8 @@ def test_command_line(model_a, capsys):
     for p, o in zip(([5, 17, 3], [9, 8, 7, 6]), rec["outputs"]):
         want, gaps = oracle.greedy(p, 6)
         assert_greedy_equal(o["output_token_ids"], want, gaps)
+        oracle.check_choices(p, o["output_token_ids"], 1e-4)
+        assert o["output_token_ids"] != [p[-1]] * 6
     assert rec["stats"]["kv_cache"]["num_blocks"] == 32
 
 

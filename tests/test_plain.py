@@ -104,6 +104,31 @@ def test_llama3_scaling_invariants():
         f_high.item(), rel=1e-6)
 
 
+def test_llama3_scaling_mid_band_value_worked_by_hand():
+    """Tiny B's one frequency between the thresholds (theta 5e5, head size 32, factor 4, low 1,
+    high 4, original length 64, so wavelengths between 16 and 64 are blended), by the rule
+    "between them (1 - s) f / factor + s f with s = (orig / wavelength - low) / (high - low)":
+
+        j = 2:  f = 500000^(-4/32) = 0.193922745,  wavelength = 2 pi / f = 32.4004557
+        orig / wavelength = 1.97528086,  s = (1.97528086 - 1) / 3 = 0.325093619
+        out = f (0.25 (1 - s) + s) = 0.193922745 * 0.493820214 = 0.0957629714
+
+    A blend that is linear in the wavelength instead (s = (64 - 32.4) / 48) gives 0.1442 and
+    passes every bound, order and continuity check above.  The plain model and the engine's
+    tables must both give the worked value; neighbours j = 1 (wavelength 14.27, kept) and j = 3
+    (73.58, divided by 4) pin the two thresholds' sides."""
+    from kvforge_amd.config.model import RopeScaling
+    from kvforge_amd.parts.positions import scaled_inv_freq
+    base = plain.rope_inv_freq(32, 500000.0)
+    out = plain.llama3_scale_inv_freq(base, 4.0, 1.0, 4.0, 64)
+    eng = scaled_inv_freq(32, 500000.0, RopeScaling("llama3", 4.0, 1.0, 4.0, 64))
+    for got in (out, eng):
+        assert got[2].item() == pytest.approx(0.0957629714, rel=2e-6)
+        assert got[1].item() == pytest.approx(500000.0 ** (-2 / 32), rel=1e-6)
+        assert got[3].item() == pytest.approx(500000.0 ** (-6 / 32) / 4.0, rel=1e-6)
+    torch.testing.assert_close(eng, out, rtol=1e-6, atol=0)
+
+
 # ------------------------------------------------------------------ attention
 @pytest.mark.parametrize("H,KV,d", [(4, 2, 16), (3, 1, 32), (4, 4, 8)])
 def test_attention_is_the_library_routine(H, KV, d):

@@ -59,7 +59,7 @@ def test_replay_all_modes(tmp_path, name, dtype, sharp):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["WIDE", "WIDE_B"])
+@pytest.mark.parametrize("which", ["WIDE", "WIDE_B", "WIDE_C"])
 def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, which):
     """The tiny configurations are below the sizes at which the bf16 engine changes kernels.
     This one is not: its down projection is cut in two halves of K for up to 16 rows, and the
@@ -73,6 +73,9 @@ def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, whic
     few = torch.empty(3, cfg["intermediate_size"], dtype=bf)
     deep = torch.empty(cfg["hidden_size"], cfg["intermediate_size"], dtype=bf)
     assert ops.k_halves_pay(few, deep) and not ops.is_library_product(few, deep)
+    if which == "WIDE_C":     # the output projection as well
+        heads = cfg["num_attention_heads"] * cfg["head_dim"]
+        assert ops.k_halves_pay(torch.empty(3, heads, dtype=bf), torch.empty(cfg["hidden_size"], heads, dtype=bf))
     folder = str(tmp_path / "model")
     kvforge_amd.write_random_model(folder, cfg, seed=4)
     prompts = ru.random_prompts(cfg["vocab_size"], [41, 75, 52, 66], 9)
@@ -80,6 +83,117 @@ def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, whic
     out = str(tmp_path / "out")
     ru.run_trace(folder, dtype, tb, out)
     ru.compare(folder, tb, out, names, *TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_tiny_b_at_its_own_pages_of_eight_tokens(tmp_path, dtype):
+    """Tiny B as its configuration has it: pages of 8 tokens (``--block-size 8``), all four ways
+    of cutting the requests, with a pool so small that pages are used again."""
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1)
+    ru.sharpen(folder, 6.0)
+    prompts = ru.random_prompts(384, [1, 9, 40, 70, 129, 57], 1)
+    tb, names = build_all_modes(prompts, 1)
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, dtype, tb, out, user_args=["--block-size", "8", "--max-live", "4"])
+    ru.compare(folder, tb, out, names, *TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_an_id_that_ends_and_comes_back_with_other_tokens(tmp_path, dtype):
+    """What preemption does to the cache, seen from the step function: request "x" is fed and
+    decodes beside "y", ends (its pages go back to the pool), "y" and a newcomer grow into those
+    pages, and "x" comes back under the same id from position 0, first with its old tokens and
+    more (recomputation), later once again with entirely different tokens, each time
+    landing in pages that others have written since.  The engine keeps, per row of the block
+    tables on the device, who the row belongs to; an id that returns must not be taken for its
+    former self.  Every logit is compared with the plain model."""
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, dict(ru.TINY_C), seed=6)
+    ru.sharpen(folder, 6.0)
+    p = ru.random_prompts(200, [90, 120, 70, 80], 21)
+    first, y, z, other = p["p0"], p["p1"], p["p2"], p["p3"]
+    every = lambda n: list(range(n))
+    tb = ru.TraceBuilder()
+    tb.step([("x", first[:40], every(40), "x1"), ("y", y[:33], every(33))])
+    for i in range(6):
+        tb.step([("x", [first[40 + i]], [0], "x1"), ("y", [y[33 + i]], [0])])
+    tb.step([("y", y[39:60], every(21))], end=["x"])                       # x loses its pages
+    tb.step([("y", y[60:100], every(40)), ("z", z[:50], every(50))])       # others grow into them
+    # x again: what it held before and ten tokens more, from position 0, as a recomputation does
+    tb.step([("y", [y[100]], [0]), ("x", first[:56], every(56), "x1"), ("z", [z[50]], [0])])
+    for i in range(8):
+        tb.step([("y", [y[101 + i]], [0]), ("x", [first[56 + i]], [0], "x1"), ("z", [z[51 + i]], [0])])
+    tb.step([("z", z[59:], every(11))], end=["x", "z"])
+    # A third life with other tokens, in the batch row x sat in last (the second), which no step
+    # has used in between, and with as many pages as it had there: only the allocation's serial
+    # number tells the engine that the row's table on the device is not this request's.
+    tb.step([("y", y[109:], every(11)), ("x", other[:64], every(64), "x2")])
+    tb.step([("x", other[64:], every(16), "x2")], end=["x", "y"])
+    names = {"x1": first, "x2": other, "y": y, "z": z}
+    out = str(tmp_path / "out")
+    # room for three live requests at most: x's pages must be among those that y and z take
+    ru.run_trace(folder, dtype, tb, out, max_tokens=tb.peak)
+    ru.compare(folder, tb, out, names, *TOL[dtype])
+
+
+SERVED = {
+    # two layers of the Llama 3.2 1B shape with its whole vocabulary (8,016 groups of 16 columns
+    # in the head), tied
+    "1b": lambda: dict(kvforge_amd.preset_dict("llama-1b"), num_hidden_layers=2,
+                       max_position_embeddings=2048),
+    # two layers of the Llama 3.1 8B layer shape: width 4096, head size 128, 14336 wide
+    # feed-forward, untied head over a vocabulary that ends inside a group of 16 columns
+    "8b": lambda: dict(kvforge_amd.preset_dict("llama-8b"), num_hidden_layers=2, vocab_size=32003,
+                       max_position_embeddings=2048),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", list(SERVED))
+def test_replay_at_the_served_width(tmp_path, shape, dtype):
+    """The bf16 engine changes kernels by size: the norm folded into the projection up to 16
+    rows, the weight-streaming kernel up to 32 (64 where its epilogue replaces a kernel), the
+    library's product beyond, two column groups per wave for wide weights, the down projection
+    in two halves of K.  Here the layers have the widths that are served, and steps of exactly
+    16, 17, 32, 33, 64 and 65 tokens stand on both sides of every threshold; all four ways of
+    cutting requests, against the plain model (some places of each step, the vocabulary being
+    large)."""
+    cfg = SERVED[shape]()
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, cfg, seed=12)
+    # At these widths q.k already spreads over a few units (its spread grows with the width);
+    # 1.5 makes the scores' spread about 2 (1B shape) and 4 (8B shape): peaked enough for one
+    # wrong key to show, without multiplying the rounding of q and k into the logits.
+    ru.sharpen(folder, 1.5)
+    prompts = ru.random_prompts(cfg["vocab_size"], [240, 80, 100, 60], 13)
+    a, b, c, d = (prompts[f"p{i}"] for i in range(4))
+    tb = ru.TraceBuilder()
+    names = {}
+    # whole
+    names["a#w"], names["b#w"] = a, b
+    tb.step([("a#w", a, [0, 15, 16, 100, 239])], end=["a#w"])
+    tb.step([("b#w", b, [0, 40, 79])], end=["b#w"])
+    # most in one step, the last 32 one by one
+    names["c#d"] = c
+    ru.decode_tail(tb, "c#d", c)
+    tb.steps[-33]["entries"][0]["want"] = [0, 33, 67]
+    tb.expect[-33] = [("c#d", 0), ("c#d", 33), ("c#d", 67)]
+    # portions on both sides of every threshold, then single tokens
+    names["a#p"] = a
+    pos = 0
+    for n in (16, 17, 32, 33, 64, 65):
+        tb.step([("a#p", a[pos:pos + n], [0, n // 2, n - 1])])
+        pos += n
+    for i in range(pos, len(a)):
+        tb.step([("a#p", [a[i]], [0])], end=["a#p"] if i == len(a) - 1 else [])
+    # mixed, pages used again
+    mixed_prompts = {"b#m": b, "c#m": c, "d#m": d, "a#m": a[:120]}
+    names.update(mixed_prompts)
+    ru.mixed(tb, mixed_prompts, 5, max_want=3)
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, dtype, tb, out)
+    ru.compare(folder, tb, out, names, *TOL[dtype], measured_rounding=True if dtype == "float32" else dtype)
 
 
 def test_replay_first_tokens_and_one_token_requests(tmp_path):

@@ -106,6 +106,42 @@ def test_tied_head_tolerates_a_stored_copy_and_untied_needs_it(tmp_path):
         Transformer.from_folder(folder_b, torch.float32, "cpu")
 
 
+def test_a_model_in_several_files_named_by_the_index(tmp_path):
+    """Two and three shards with ``model.safetensors.index.json``: the loader finds every tensor
+    by name whichever file holds it, the model is bit for bit the one-file model, and an index
+    that names a file that is not there is one clear error."""
+    import json
+    import os
+    folder = make(tmp_path, "tiny-b", 1)
+    w = read_safetensors_folder(folder)
+    one = Transformer.from_folder(folder, torch.float32, "cpu")
+    for shards in (2, 3):
+        sharded = str(tmp_path / f"shards{shards}")
+        registry.config_from_dict(preset_dict("tiny-b")).save(sharded)
+        index = write_safetensors(sharded, w, shards=shards)
+        with open(index) as f:
+            weight_map = json.load(f)["weight_map"]
+        files = sorted(set(weight_map.values()))
+        assert len(files) == shards and set(weight_map) == set(w)
+        assert not os.path.exists(os.path.join(sharded, "model.safetensors"))
+        # layers are spread over the files, so a loader that read one file would miss some
+        assert len({weight_map[n] for n in w if ".layers." in n}) > 1
+        back = read_safetensors_folder(sharded)
+        assert set(back) == set(w) and all(torch.equal(back[k], w[k]) for k in w)
+        many = Transformer.from_folder(sharded, torch.float32, "cpu")
+        for a, b in zip(one.spec.blocks, many.spec.blocks):
+            assert torch.equal(a.mixer.w_qkv, b.mixer.w_qkv) and torch.equal(a.ffn.w_down, b.ffn.w_down)
+        assert torch.equal(one.spec.head.weight, many.spec.head.weight)
+    # a tensor missing from every shard is reported like any missing tensor
+    del w["model.layers.2.mlp.down_proj.weight"]
+    write_safetensors(sharded, w, shards=3)
+    with pytest.raises(WeightsError, match="model.layers.2.mlp.down_proj.weight"):
+        Transformer.from_folder(sharded, torch.float32, "cpu")
+    os.remove(os.path.join(sharded, files[1]))
+    with pytest.raises(WeightsError, match=files[1]):
+        Transformer.from_folder(sharded, torch.float32, "cpu")
+
+
 def test_missing_files(tmp_path):
     with pytest.raises(kvforge_amd.ConfigError):
         Transformer.from_folder(str(tmp_path), torch.float32, "cpu")
