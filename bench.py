@@ -12,6 +12,12 @@ N(0, 0.02), batch 8, 512-token uniform-random prompts, greedy, context cap 8192,
 tokens.  A step is one decode step of the whole engine (scheduler, batch building, forward,
 sampling, bookkeeping).  One JSON line is printed; besides the decode figure it carries a
 2,048-token prefill, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+``points`` also holds (unless ``--no-points``) the same model in true 32-bit (decode at batch 1
+and 8, prefill of 2,048 tokens, with their shares of the fp32 bounds), the mixed workload at the
+Llama 3.2 3B shape (32 requests, prompts of 128 to 4,096 tokens, chunked prefill under a
+2,048-token budget beside decode steps, 256 new tokens each) and long-context decoding at the
+Llama 3.1 8B shape, all 32 layers (batch 16 at 32,768-token prompts, 128 new tokens); these two
+draw their random weights on the device.
 Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
 for fp32.
 """
@@ -44,8 +50,10 @@ SMALL = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_si
          "tie_word_embeddings": False}
 
 
-def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True, run_steps=None,
+def build_engine(model, dtype, max_num_seqs, num_tokens_cached, use_graphs=True, run_steps=None,
                  context_cap=CONTEXT_CAP):
+    """``model``: a model folder, or a config.json dictionary whose random weights are drawn on
+    the device."""
     import kvforge_amd
     from kvforge_amd import CacheConfig, EngineConfig, InferenceEngine, SchedulerConfig
 
@@ -57,7 +65,9 @@ def build_engine(folder, dtype, max_num_seqs, num_tokens_cached, use_graphs=True
         dtype=dtype, use_graphs=use_graphs)
     if run_steps is not None:
         cfg.decode_run_steps = run_steps
-    return InferenceEngine.from_folder(folder, cfg)
+    if isinstance(model, dict):
+        return InferenceEngine.from_config(model, cfg, on_device=True)
+    return InferenceEngine.from_folder(model, cfg)
 
 
 def random_prompts(vocab, n, length, seed):
@@ -150,11 +160,14 @@ def mixed_run(engine, vocab, requests, new_tokens, seed=0):
     prompts = [torch.randint(1, vocab, (n,), generator=g).tolist() for n in lens]
     params = SamplingParams(max_tokens=new_tokens, temperature=0.0, ignore_eos=True)
     engine.generate(prompts[:2], SamplingParams(max_tokens=24, temperature=0.0, ignore_eos=True))  # warm-up
+    engine.metrics.reset()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     outs = engine.generate(prompts, params)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    mixed_run.last = {"lens": lens, "steps": engine.metrics.num_steps,
+                      "step_tokens": list(engine.metrics.batched_tokens)}
     return sum(lens), sum(len(o.output_token_ids) for o in outs), dt
 
 
@@ -194,6 +207,90 @@ def burst_run(folder, vocab, dtype, use_graphs, seed=0):
     return sum(lens), best
 
 
+def decode_bytes(engine, nums, elem, batch, mean_ctx):
+    """What a decode step has to read: every weight it uses once, and the cache of the live
+    requests."""
+    return engine.model.weight_bytes + batch * mean_ctx * nums["kv_values_per_token"] * elem
+
+
+def prefill_flops(nums, n):
+    """Linear layers over ``n`` tokens, the head for one row, causal attention."""
+    return (2.0 * n * nums["linear_params"] + 2.0 * nums["head_params"]
+            + 2.0 * n * n * nums["attn_hd"] * nums["layers"])
+
+
+def fp32_points(folder, cfg, vocab, nums, steps=48, warmup=8):
+    """The 1B shape in true 32-bit: decode at batch 1 and 8, prefill of 2,048 tokens."""
+    import torch
+    out = {}
+    for b in (8, 1):
+        need = b * (512 + steps + warmup + early_tokens(b, 512) + 32)
+        engine = build_engine(folder, "float32", b, max(need, PREFILL_TOKENS + 64))
+        r = decode_run(engine, vocab, b, 512, steps, warmup)
+        out[f"fp32_decode_b{b}"] = round(r["tok_s"], 1)
+        out[f"fp32_decode_b{b}_ms"] = round(r["ms_per_step"], 4)
+        out[f"fp32_decode_b{b}_hbm_frac"] = round(
+            decode_bytes(engine, nums, 4, b, r["mean_ctx"]) / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4)
+        if b == 8:
+            s = prefill_run(engine, vocab, PREFILL_TOKENS, repeats=2)
+            out["fp32_prefill_tok_s"] = round(PREFILL_TOKENS / s, 1)
+            out["fp32_prefill_ms"] = round(s * 1e3, 3)
+            out["fp32_prefill_frac"] = round(prefill_flops(nums, PREFILL_TOKENS) / s / MFMA_PEAK["float32"], 4)
+        del engine
+        torch.cuda.empty_cache()
+    return out
+
+
+def mixed_3b_points(requests=32, new_tokens=256):
+    """BASELINE's mixed workload at the Llama 3.2 3B shape, bf16."""
+    import torch
+    import kvforge_amd
+    cfg = kvforge_amd.preset_dict("llama-3b")
+    nums = model_numbers(cfg, cfg["num_hidden_layers"])
+    engine = build_engine(cfg, "bfloat16", requests, requests * (4096 + new_tokens + 64))
+    prompt_tokens, generated, dt = mixed_run(engine, cfg["vocab_size"], requests, new_tokens)
+    info = mixed_run.last
+    flops = 2.0 * nums["linear_params"] * (prompt_tokens + generated)
+    cache_read = 0.0
+    per_token = nums["kv_values_per_token"] * 2
+    for n in info["lens"]:
+        flops += 2.0 * n * n * nums["attn_hd"] * nums["layers"]                      # the prompt, causal
+        flops += 4.0 * new_tokens * (n + new_tokens / 2) * nums["attn_hd"] * nums["layers"]
+        cache_read += new_tokens * (n + new_tokens / 2) * per_token                  # decode steps
+    read = info["steps"] * engine.model.weight_bytes + cache_read
+    out = {"mixed_3b_tok_s": round((prompt_tokens + generated) / dt, 1),
+           "mixed_3b_gen_tok_s": round(generated / dt, 1), "mixed_3b_s": round(dt, 4),
+           "mixed_3b_steps": info["steps"], "mixed_3b_ms_per_step": round(dt / info["steps"] * 1e3, 4),
+           "mixed_3b_mfma_frac": round(flops / dt / MFMA_PEAK["bfloat16"], 4),
+           "mixed_3b_hbm_frac": round(read / dt / 1e9 / HBM_PEAK_GBS, 4)}
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
+def long_8b_points(batch=16, prompt_len=32768, new_tokens=128, warmup=8):
+    """BASELINE's long-context decode at the Llama 3.1 8B shape, all 32 layers, bf16."""
+    import torch
+    import kvforge_amd
+    cfg = kvforge_amd.preset_dict("llama-8b")
+    nums = model_numbers(cfg, cfg["num_hidden_layers"])
+    steps = new_tokens - 1
+    need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
+    engine = build_engine(cfg, "bfloat16", batch, need, context_cap=prompt_len + 1024)
+    t0 = time.perf_counter()
+    r = decode_run(engine, cfg["vocab_size"], batch, prompt_len, steps, warmup)
+    total = time.perf_counter() - t0
+    read = decode_bytes(engine, nums, 2, batch, r["mean_ctx"])
+    out = {"long_8b_tok_s": round(r["tok_s"], 1), "long_8b_ms_per_step": round(r["ms_per_step"], 4),
+           "long_8b_hbm_frac": round(read / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
+           "long_8b_layers": cfg["num_hidden_layers"], "long_8b_batch": batch,
+           "long_8b_context": int(r["mean_ctx"]), "long_8b_steps": steps,
+           "long_8b_prefill_tok_s": round(batch * prompt_len / max(total - r["seconds"], 1e-9), 1)}
+    del engine
+    torch.cuda.empty_cache()
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -215,7 +312,10 @@ def main() -> int:
     ap.add_argument("--context-len", type=int, default=CONTEXT_CAP,
                     help="longest request the engine admits (prompt and new tokens)")
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
-    ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true",
+                    help="skip decode at batch 1 and 64, the 32-bit run and the 3B and 8B workloads")
+    ap.add_argument("--only-points", default=None,
+                    help="comma-separated subset of fp32,mixed_3b,long_8b to run besides the main line")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
@@ -287,6 +387,19 @@ def main() -> int:
                 weight_bytes = engine.model.weight_bytes
             del engine
             torch.cuda.empty_cache()
+        more = {}
+        if points and args.preset == "llama-1b" and layers_run == full_layers:
+            chosen = set((args.only_points or "fp32,mixed_3b,long_8b").split(","))
+            for name, fn in (("fp32", lambda: fp32_points(folder, cfg, vocab, nums)),
+                             ("mixed_3b", mixed_3b_points), ("long_8b", long_8b_points)):
+                if name not in chosen:
+                    continue
+                try:
+                    more.update(fn())
+                except Exception as e:   # the main line is printed whatever happens to an extra
+                    print(f"bench: {name} failed: {type(e).__name__}: {e}", file=sys.stderr)
+                    more[f"{name}_failed"] = 1
+                    torch.cuda.empty_cache()
 
     if args.phase != "all":  # a partial run for a profile: say what was timed and stop
         part = ({"prefill_ms": round(prefill_s * 1e3, 3)} if args.phase == "prefill" else
@@ -299,8 +412,6 @@ def main() -> int:
     kv_bytes = args.batch * main_run["mean_ctx"] * nums["kv_values_per_token"] * elem
     achieved = (weight_bytes + kv_bytes) / step_s / 1e9
     n = PREFILL_TOKENS
-    prefill_flops = (2.0 * n * nums["linear_params"] + 2.0 * nums["head_params"]
-                     + 2.0 * n * n * nums["attn_hd"] * layers_run)
     line = {
         "metric": "decode tok/s (%s shape, batch %d)" % (MODEL_NAMES[args.preset], args.batch),
         "value": round(main_run["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1,
@@ -320,10 +431,11 @@ def main() -> int:
             "sampling": "greedy", "decode_run_steps": run_steps_used,
         },
         "prefill": {"value": round(n / prefill_s, 1), "tokens": n, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(prefill_flops / prefill_s / MFMA_PEAK[args.dtype], 4)},
+                    "frac": round(prefill_flops(nums, n) / prefill_s / MFMA_PEAK[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
-        "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+        "points": {**{f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+                   **more},
     }
     print(json.dumps(line))
     return 0

@@ -60,13 +60,20 @@ class InferenceEngine:
 
     @classmethod
     def from_config(cls, model_config: "dict[str, Any] | str", config: EngineConfig | None = None,
-                    tokenizer: Any = None, seed: int | None = None) -> "InferenceEngine":
+                    tokenizer: Any = None, seed: int | None = None,
+                    on_device: bool = False) -> "InferenceEngine":
         """Random weights: ``model_config`` is a config.json dictionary or a preset name; the
-        model folder is written to a temporary place and loaded like any other."""
+        model folder is written to a temporary place and loaded like any other.  With
+        ``on_device`` the tensors are drawn on the GPU instead and no file is written (for
+        models of many gigabytes; other numbers than the folder's for the same seed)."""
         from kvforge_amd.config.presets import preset_dict
 
         config = config or EngineConfig()
         d = preset_dict(model_config) if isinstance(model_config, str) else model_config
+        if on_device:
+            model = Transformer.from_random(d, config.seed if seed is None else seed, config.dtype,
+                                            config.device)
+            return cls(model, config, tokenizer)
         with tempfile.TemporaryDirectory(prefix="kvforge_amd_model_") as tmp:
             write_random_model(tmp, d, config.seed if seed is None else seed)
             return cls.from_folder(tmp, config, tokenizer)

@@ -57,6 +57,21 @@ class Transformer:
         model.load_folder(folder)
         return model
 
+    @classmethod
+    def from_random(cls, config, seed: int, dtype: torch.dtype, device: torch.device | str = "cuda"
+                    ) -> "Transformer":
+        """Random weights drawn on the device, no files (``config``: a config.json dictionary or
+        a typed configuration)."""
+        from kvforge_amd.weights.random_init import load_random_weights
+
+        cfg = registry.config_from_dict(config) if isinstance(config, dict) else config
+        model = cls(registry.build_spec(cfg), dtype, device)
+        load_random_weights(model.spec, seed, dtype, device)
+        for p in model.spec.all_parts():
+            p.seal()
+        model._loaded = True
+        return model
+
     def load_folder(self, folder: str) -> None:
         load_model_weights(self.spec, folder, self.dtype, self.device)
         for p in self.spec.all_parts():

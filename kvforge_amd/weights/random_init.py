@@ -47,3 +47,32 @@ def write_random_model(folder: str, config: "dict[str, Any] | Any", seed: int = 
     cfg.save(folder)
     write_safetensors(folder, random_tensors(spec, seed, dtype))
     return folder
+
+
+def load_random_weights(spec, seed: int, engine_dtype: torch.dtype, device: "torch.device | str",
+                        dtype: str = "bfloat16") -> None:
+    """The random-weights mode without the files, for models too large to be worth writing:
+    every tensor of ``spec`` is drawn on ``device`` (same laws, same name order, stored in
+    ``dtype`` and then held as the loader would hold a tensor stored so) and handed to the
+    parts.  The device's generator gives other numbers than ``write_random_model`` does for the
+    same seed."""
+    from kvforge_amd.weights.loader import runtime_dtype
+
+    store = _STORE[dtype]
+    gen = torch.Generator(device=device).manual_seed(int(seed))
+    tensors: dict[str, torch.Tensor] = {}
+    for name, w in sorted(spec.weight_specs().items()):
+        if w.integer:
+            tensors[name] = torch.zeros(w.shape, dtype=torch.int32, device=device)
+            continue
+        if w.init == "zeros":
+            t = torch.zeros(w.shape, dtype=torch.float32, device=device)
+        elif w.init in ("normal", "norm"):
+            t = torch.randn(w.shape, generator=gen, dtype=torch.float32, device=device) * w.std
+            if w.init == "norm":
+                t += 1.0
+        else:
+            raise ValueError(f"unknown init {w.init!r} for {name}")
+        tensors[name] = t.to(store).to(runtime_dtype(store, engine_dtype)).contiguous()
+    for part in spec.all_parts():
+        part.load(tensors)
