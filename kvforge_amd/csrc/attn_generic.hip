@@ -196,7 +196,293 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
 #undef GO
   return kvf_last_error();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Single-token queries (decode steps).  A workgroup of four waves takes one (sequence, kv head,
+// cut of the key range); its waves take blocks of 64 keys in turn.  For the scores a lane owns
+// one key and reads that key's row of the K page 16 bytes at a time, against the queries of all
+// heads of the group (held in LDS, read as broadcasts), so K is read once for the group.  For
+// the output a lane owns elements lane, lane + 64, ... of the head and walks the block's keys
+// through the transposed V page, four keys per load, the probabilities again as broadcasts
+// from LDS.  Running maximum, sum and accumulator per head are merged over the four waves in
+// LDS, and over the cuts (when there are several) by attn_decode_merge_kernel from fp32
+// partial results; the order of every sum is fixed by the shapes.
+constexpr int DEC_WAVES = 4, DEC_KEYS = 64;
+
+struct DecodeArgs {
+  int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs, splits;
+  float scale;
+};
+
+// GT: heads of the group handled together (a power of two, at most 8; a larger group is taken
+// in chunks of 8 heads by workgroups of their own); DQ: elements of the head per lane
+// (ceil(d / 64)).
+template <typename T, int GT, int DQ>
+__global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int* __restrict__ block_table, const int* __restrict__ seq_ids,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, T* __restrict__ out,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, DecodeArgs a) {
+  __shared__ float Qs[GT][256];
+  __shared__ float Ps[DEC_WAVES][GT][DEC_KEYS];
+  __shared__ float Ms[DEC_WAVES][GT], Ls[DEC_WAVES][GT];
+  __shared__ float Os[DEC_WAVES][GT][DQ * KVF_WAVE];
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE;
+  const int G = a.H / a.KV, D = a.d;
+  const int chunks = (G + GT - 1) / GT;
+  const int kvh = blockIdx.x / chunks, g0 = (blockIdx.x % chunks) * GT;
+  const int cut = blockIdx.y, slot = blockIdx.z;
+  const int seq = seq_ids ? seq_ids[slot] : slot;
+  const bool seq_ok = seq >= 0 && seq < a.n_seqs;
+  const int ctx = seq_ok ? ctx_lens[seq] : 0;
+  const int token = seq_ok ? (cu_q ? cu_q[seq] : seq) : 0;
+  const int pos = ctx - 1;
+  int lo = 0;
+  if (a.window > 0 && pos - a.window + 1 > 0) lo = pos - a.window + 1;
+  // blocks of 64 keys from the block that holds `lo`; this cut takes blocks [b_lo, b_hi)
+  const int first = lo / DEC_KEYS;
+  const int n_blocks = ctx > 0 ? pos / DEC_KEYS - first + 1 : 0;
+  const int per_cut = (n_blocks + a.splits - 1) / a.splits;
+  const int b_lo = first + cut * per_cut, b_hi = min(first + n_blocks, b_lo + per_cut);
+  const int* table = block_table + static_cast<size_t>(seq_ok ? seq : 0) * a.table_stride;
+
+  for (int idx = tid; idx < GT * D; idx += DEC_WAVES * KVF_WAVE) {
+    const int g = idx / D, kk = idx - g * D;
+    Qs[g][kk] = (g0 + g < G && ctx > 0)
+                    ? Elem<T>::load(q + static_cast<size_t>(token) * a.q_stride + (kvh * G + g0 + g) * D + kk)
+                    : 0.f;
+  }
+  __syncthreads();
+
+  float m_run[GT], l_run[GT], acc[GT][DQ];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    m_run[g] = -INFINITY;
+    l_run[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < DQ; ++i) acc[g][i] = 0.f;
+  }
+  const bool quads = a.block_size % 4 == 0;
+  for (int b = b_lo + wave; b < b_hi; b += DEC_WAVES) {
+    const int j = b * DEC_KEYS + lane;  // this lane's key
+    const bool vis = j >= lo && j <= pos;
+    // the page of every key of the context, visible or not: the values of four neighbouring keys
+    // are read together further down, and a hidden one among them only has probability zero
+    int page = -1;
+    if (j <= pos) {
+      const int blk = j / a.block_size;
+      page = blk < a.table_stride ? table[blk] : -1;
+      if (page >= a.num_blocks) page = -1;
+    }
+    const int off = j % a.block_size;
+    float s[GT];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) s[g] = 0.f;
+    if (vis && page >= 0) {
+      const T* krow = k_pages + ((static_cast<size_t>(page) * a.KV + kvh) * a.block_size + off) * D;
+      for (int kc = 0; kc < D; kc += 16) {
+        float kv[16];
+        load8(krow + kc, *reinterpret_cast<float(*)[8]>(&kv[0]));
+        load8(krow + kc + 8, *reinterpret_cast<float(*)[8]>(&kv[8]));
+#pragma unroll
+        for (int g = 0; g < GT; ++g) {
+          float t = s[g];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) t = fmaf(Qs[g][kc + e], kv[e], t);
+          s[g] = t;
+        }
+      }
+    }
+    float corr[GT];
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      const float sc = (vis && page >= 0) ? s[g] * a.scale : -INFINITY;
+      const float m_new = fmaxf(m_run[g], wave_max(sc));
+      float p = 0.f;
+      corr[g] = 1.f;
+      if (m_new > -INFINITY) {
+        corr[g] = expf(m_run[g] - m_new);  // 0 on the first block with a visible key
+        p = expf(sc - m_new);
+      }
+      Ps[wave][g][lane] = p;
+      l_run[g] = l_run[g] * corr[g] + wave_sum(p);
+      m_run[g] = m_new;
+#pragma unroll
+      for (int i = 0; i < DQ; ++i) acc[g][i] *= corr[g];
+    }
+    // ---- output: elements lane + 64 i over the block's keys
+    const int step = quads ? 4 : 1;
+    for (int c = 0; c < DEC_KEYS; c += step) {
+      // keys c .. c+3 share a page when pages hold a multiple of four; no page: the keys lie
+      // beyond the context or in a page that a window has given back
+      const int pg = __shfl(page, c, KVF_WAVE);
+      if (pg < 0) continue;
+      const int o = (b * DEC_KEYS + c) % a.block_size;
+#pragma unroll
+      for (int i = 0; i < DQ; ++i) {
+        const int e = lane + KVF_WAVE * i;
+        if (e >= D) continue;
+        const T* vp = v_pages + ((static_cast<size_t>(pg) * a.KV + kvh) * D + e) * a.block_size + o;
+        if (quads) {
+          float v4[4];
+          if (sizeof(T) == 4) {
+            const float4 r = *reinterpret_cast<const float4*>(vp);
+            v4[0] = r.x; v4[1] = r.y; v4[2] = r.z; v4[3] = r.w;
+          } else {
+            const uint2 r = *reinterpret_cast<const uint2*>(vp);
+            v4[0] = __uint_as_float(r.x << 16); v4[1] = __uint_as_float(r.x & 0xffff0000u);
+            v4[2] = __uint_as_float(r.y << 16); v4[3] = __uint_as_float(r.y & 0xffff0000u);
+          }
+#pragma unroll
+          for (int g = 0; g < GT; ++g) {
+            float t = acc[g][i];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) t = fmaf(Ps[wave][g][c + x], v4[x], t);  // hidden keys have p = 0
+            acc[g][i] = t;
+          }
+        } else {
+          const float v = Elem<T>::load(vp);
+#pragma unroll
+          for (int g = 0; g < GT; ++g) acc[g][i] = fmaf(Ps[wave][g][c], v, acc[g][i]);
+        }
+      }
+    }
+  }
+  // ---- the four waves' results into one
+  if (lane < GT) {
+    float mv = -INFINITY, lv = 0.f;
+#pragma unroll
+    for (int g = 0; g < GT; ++g)
+      if (g == lane) { mv = m_run[g]; lv = l_run[g]; }
+    Ms[wave][lane] = mv;
+    Ls[wave][lane] = lv;
+  }
+#pragma unroll
+  for (int g = 0; g < GT; ++g)
+#pragma unroll
+    for (int i = 0; i < DQ; ++i) Os[wave][g][lane + KVF_WAVE * i] = acc[g][i];
+  __syncthreads();
+  if (!seq_ok) return;
+  for (int idx = tid; idx < min(GT, G - g0) * D; idx += DEC_WAVES * KVF_WAVE) {
+    const int g = idx / D, e = idx - g * D;
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) m = fmaxf(m, Ms[w][g]);
+    float l = 0.f, o = 0.f;
+    if (m > -INFINITY) {
+#pragma unroll
+      for (int w = 0; w < DEC_WAVES; ++w) {
+        const float f = expf(Ms[w][g] - m);   // exp(-inf) = 0 for a wave that saw no key
+        l += Ls[w][g] * f;
+        o += Os[w][g][e] * f;
+      }
+    }
+    const int head = kvh * G + g0 + g;
+    if (a.splits == 1) {
+      if (ctx > 0)
+        Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * D + e,
+                       l > 0.f ? o / l : 0.f);
+    } else {
+      const size_t p = (static_cast<size_t>(slot) * a.H + head) * a.splits + cut;
+      part_acc[p * D + e] = o;
+      if (e == 0) {
+        part_ml[2 * p] = m;
+        part_ml[2 * p + 1] = l;
+      }
+    }
+  }
+}
+
+// One workgroup per (sequence slot, head): the cuts' partial results into the output row, in
+// cut order.  A sequence without context (padding of a captured batch) writes nothing.
+template <typename T>
+__global__ __launch_bounds__(KVF_WAVE) void attn_decode_merge_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    T* __restrict__ out, DecodeArgs a) {
+  const int head = blockIdx.x, slot = blockIdx.y;
+  const int seq = seq_ids ? seq_ids[slot] : slot;
+  if (seq < 0 || seq >= a.n_seqs || ctx_lens[seq] <= 0) return;
+  const int token = cu_q ? cu_q[seq] : seq;
+  const size_t p0 = (static_cast<size_t>(slot) * a.H + head) * a.splits;
+  float m = -INFINITY;
+  for (int c = 0; c < a.splits; ++c) m = fmaxf(m, part_ml[2 * (p0 + c)]);
+  for (int e = threadIdx.x; e < a.d; e += KVF_WAVE) {
+    float l = 0.f, o = 0.f;
+    if (m > -INFINITY) {
+      for (int c = 0; c < a.splits; ++c) {
+        const float f = expf(part_ml[2 * (p0 + c)] - m);
+        l += part_ml[2 * (p0 + c) + 1] * f;
+        o += part_acc[(p0 + c) * a.d + e] * f;
+      }
+    }
+    Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * a.d + e, l > 0.f ? o / l : 0.f);
+  }
+}
+
+template <typename T, int GT>
+int launch_decode_g(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                    const int* seq_ids, const int* cu_q, const int* ctx_lens, void* out,
+                    float* part_acc, float* part_ml, int num_seqs, DecodeArgs a, hipStream_t s) {
+  const int G = a.H / a.KV;
+  dim3 grid(a.KV * ((G + GT - 1) / GT), a.splits, num_seqs);
+#define GO(DQ)                                                                                    \
+  hipLaunchKernelGGL((attn_decode_kernel<T, GT, DQ>), grid, dim3(DEC_WAVES * KVF_WAVE), 0, s,     \
+                     static_cast<const T*>(q), static_cast<const T*>(k_pages),                    \
+                     static_cast<const T*>(v_pages), block_table, seq_ids, cu_q, ctx_lens,        \
+                     static_cast<T*>(out), part_acc, part_ml, a)
+  if (a.d <= 64) GO(1);
+  else if (a.d <= 128) GO(2);
+  else GO(4);
+#undef GO
+  int code = kvf_last_error();
+  if (code != 0 || a.splits == 1) return code;
+  hipLaunchKernelGGL((attn_decode_merge_kernel<T>), dim3(a.H, num_seqs), dim3(KVF_WAVE), 0, s, part_acc,
+                     part_ml, seq_ids, cu_q, ctx_lens, static_cast<T*>(out), a);
+  return kvf_last_error();
+}
+
+template <typename T>
+int launch_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                  const int* seq_ids, const int* cu_q, const int* ctx_lens, void* out,
+                  float* part_acc, float* part_ml, int num_seqs, DecodeArgs a, hipStream_t s) {
+  const int G = a.H / a.KV;
+#define GO(GT)                                                                                     \
+  return launch_decode_g<T, GT>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,    \
+                                part_acc, part_ml, num_seqs, a, s)
+  if (G <= 1) GO(1);
+  if (G <= 2) GO(2);
+  if (G <= 4) GO(4);
+  GO(8);
+#undef GO
+}
 }  // namespace
+
+// Single-token queries: sequence slots 0..num_seqs-1 are the sequences seq_ids[slot] (or the
+// slots themselves when seq_ids is null); a sequence's token is cu_q[seq] (or seq when cu_q is
+// null).  splits > 1 cuts every key range into that many runs of whole blocks of 64 keys and
+// needs part_acc (num_seqs * H * splits * d floats) and part_ml (num_seqs * H * splits * 2).
+KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_pages,
+                                       const void* v_pages, const int* block_table,
+                                       const int* seq_ids, const int* cu_q, const int* ctx_lens,
+                                       void* out, float* part_acc, float* part_ml, int num_seqs,
+                                       int H, int KV, int d, int block_size, int num_blocks,
+                                       int table_stride, int q_stride, int o_stride, int window,
+                                       int n_seqs, int splits, float scale, hipStream_t s) {
+  if (num_seqs <= 0) return 0;
+  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
+      (splits > 1 && (!part_acc || !part_ml)) || block_size <= 0)
+    return static_cast<int>(hipErrorInvalidValue);
+  DecodeArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
+               splits, scale};
+  if (dtype == 0)
+    return launch_decode<float>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
+                                part_acc, part_ml, num_seqs, a, s);
+  if (dtype == 1)
+    return launch_decode<bf16_t>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
+                                 part_acc, part_ml, num_seqs, a, s);
+  return static_cast<int>(hipErrorInvalidValue);
+}
 
 // dtype: 0 = fp32, 1 = bf16.  d must be a multiple of 16 and at most 256 (checked by the caller
 // and here).  tiles_per_seq == 0: `work` holds num_work rows (sequence, 16-row tile, tile or -1).

@@ -3,8 +3,14 @@
 // MFMA kernels do not take (for instance a weight that the checkpoint stores in fp32 while
 // activations are bf16).  No reduced-precision matrix instruction is used.
 //
-// Each output element is accumulated over k = 0..K-1 in one fixed order by one thread, so a
-// row's result does not depend on M, on the row's place in the batch or on the grid.
+// Two kernels.  Many rows (a portion of a prompt): tiles of 64 x 64 outputs, every output summed
+// over k = 0..K-1 in that order by one thread.  Few rows (decode steps), where the product is
+// bound by reading W once: a wave owns four columns of W for all rows, its lanes walk K side by
+// side with 16-byte loads (a wave reads 1 KB of a row of W at a time, several such loads in
+// flight), every lane keeps a partial sum per output and the 64 partial sums are added in a fixed
+// tree at the end.  Within either kernel a row's result does not depend on the number of rows, on
+// the row's place in the batch or on the grid; between the two the order of the sums differs, so
+// results agree to rounding.
 //
 // Output modes: 0 = store as TO;  1 = add into a fp32 matrix (the residual stream).
 #include "common.h"
@@ -139,10 +145,141 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A
   }
 }
 
+// ---- few rows, W streamed once: see the head of the file.
+constexpr int SW = 4;        // waves per workgroup
+constexpr int SKC = 1024;    // elements of K per staged chunk of A
+constexpr int SQ = 4 * KVF_WAVE;  // elements of K a wave reads per step (16 bytes a lane)
+
+template <typename T> struct Quad;
+template <> struct Quad<float> {
+  static __device__ __forceinline__ float4 load(const float* p) { return *reinterpret_cast<const float4*>(p); }
+};
+template <> struct Quad<bf16_t> {
+  static __device__ __forceinline__ float4 load(const bf16_t* p) {
+    const uint2 r = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                       __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u));
+  }
+};
+
+// MT rows per workgroup (1, 2, 4, 8 or 16); SN columns of W per wave, each read DEPTH steps
+// ahead, so that SN * DEPTH loads of 16 bytes are in flight per lane: narrow outputs (few
+// columns, hence few waves) take one column per wave and look far ahead, wide ones four columns.
+// The sums do not depend on MT, SN or DEPTH.  Needs K % 4 == 0 and rows of A and W that start on
+// 16 bytes (8 for bf16): the caller checks.
+template <typename TA, typename TW, typename TO, int MODE, int MT, int SN, int DEPTH>
+__global__ __launch_bounds__(SW * KVF_WAVE) void gemm_stream_kernel(
+    const TA* __restrict__ A, const TW* __restrict__ W, TO* __restrict__ C, int M, int N, int K,
+    int lda, int ldc) {
+  __shared__ __align__(16) float As[MT][SKC];
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE;
+  const int n0 = (blockIdx.x * SW + wave) * SN, m0 = blockIdx.y * MT;
+  float acc[MT][SN];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < SN; ++j) acc[i][j] = 0.f;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  // rows of W this wave reads; columns past N read row N - 1 and are dropped at the end
+  const TW* wrow[SN];
+#pragma unroll
+  for (int j = 0; j < SN; ++j) wrow[j] = W + static_cast<size_t>(min(n0 + j, N - 1)) * K + lane * 4;
+
+  float4 w[DEPTH][SN];   // w[t % DEPTH]: step t of this wave's walk along K
+#pragma unroll
+  for (int t = 0; t < DEPTH; ++t)
+#pragma unroll
+    for (int j = 0; j < SN; ++j) w[t][j] = t * SQ + lane * 4 < K ? Quad<TW>::load(wrow[j] + t * SQ) : zero;
+
+  const int steps = (K + SQ - 1) / SQ;
+  for (int t0 = 0; t0 < steps; t0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const int t = t0 + u, k = t * SQ;      // uniform
+      if (k >= K) break;
+      if (k % SKC == 0) {
+        __syncthreads();  // the chunk before has been read by every wave
+        for (int idx = tid; idx < MT * (SKC / 4); idx += SW * KVF_WAVE) {
+          const int row = idx / (SKC / 4), kq = k + (idx % (SKC / 4)) * 4;
+          float4 a = zero;
+          if (m0 + row < M && kq < K) a = Quad<TA>::load(A + static_cast<size_t>(m0 + row) * lda + kq);
+          *reinterpret_cast<float4*>(&As[row][kq - k]) = a;
+        }
+        __syncthreads();
+      }
+      float4 cur[SN];
+#pragma unroll
+      for (int j = 0; j < SN; ++j) cur[j] = w[u][j];
+      const int ahead = k + DEPTH * SQ;
+#pragma unroll
+      for (int j = 0; j < SN; ++j) w[u][j] = ahead + lane * 4 < K ? Quad<TW>::load(wrow[j] + ahead) : zero;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const float4 a = *reinterpret_cast<const float4*>(&As[i][k % SKC + lane * 4]);
+#pragma unroll
+        for (int j = 0; j < SN; ++j) {
+          float v = acc[i][j];
+          v = fmaf(a.x, cur[j].x, v);
+          v = fmaf(a.y, cur[j].y, v);
+          v = fmaf(a.z, cur[j].z, v);
+          v = fmaf(a.w, cur[j].w, v);
+          acc[i][j] = v;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < SN; ++j) {
+      const float total = wave_sum(acc[i][j]);
+      const int m = m0 + i, n = n0 + j;
+      if (lane == 0 && m < M && n < N) {
+        TO* o = C + static_cast<size_t>(m) * ldc + n;
+        if (MODE == 1) {
+          Elem<TO>::store(o, Elem<TO>::load(o) + total);
+        } else {
+          Elem<TO>::store(o, total);
+        }
+      }
+    }
+}
+
+template <typename TA, typename TW, typename TO, int MODE, int MT>
+int launch_stream(const TA* A, const TW* W, TO* C, int M, int N, int K, int lda, int ldc, hipStream_t s) {
+#define GO(SN, DEPTH)                                                                            \
+  do {                                                                                           \
+    dim3 grid((N + SN * SW - 1) / (SN * SW), (M + MT - 1) / MT);                                 \
+    hipLaunchKernelGGL((gemm_stream_kernel<TA, TW, TO, MODE, MT, SN, DEPTH>), grid,              \
+                       dim3(SW * KVF_WAVE), 0, s, A, W, C, M, N, K, lda, ldc);                   \
+  } while (0)
+  // about four waves or more per compute unit's SIMD at the widest choice that allows it
+  if (N >= 16384) GO(4, 2);
+  else if (N >= 6144) GO(2, 4);
+  else GO(1, 8);
+#undef GO
+  return kvf_last_error();
+}
+
+constexpr int STREAM_MAX_M = 32;
+
 template <typename TA, typename TW, typename TO, int MODE>
 int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
            hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
+  const bool quads = K % 4 == 0 && lda % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(A) % (4 * sizeof(TA)) == 0 &&
+                     reinterpret_cast<uintptr_t>(W) % (4 * sizeof(TW)) == 0;
+  if (M <= STREAM_MAX_M && quads) {
+    const TA* a = static_cast<const TA*>(A);
+    const TW* w = static_cast<const TW*>(W);
+    TO* c = static_cast<TO*>(C);
+    if (M == 1) return launch_stream<TA, TW, TO, MODE, 1>(a, w, c, M, N, K, lda, ldc, s);
+    if (M == 2) return launch_stream<TA, TW, TO, MODE, 2>(a, w, c, M, N, K, lda, ldc, s);
+    if (M <= 4) return launch_stream<TA, TW, TO, MODE, 4>(a, w, c, M, N, K, lda, ldc, s);
+    if (M <= 8) return launch_stream<TA, TW, TO, MODE, 8>(a, w, c, M, N, K, lda, ldc, s);
+    return launch_stream<TA, TW, TO, MODE, 16>(a, w, c, M, N, K, lda, ldc, s);
+  }
   if (M <= 2 * RM) {
     dim3 rows_grid((N + RN - 1) / RN, (M + RM - 1) / RM);
     hipLaunchKernelGGL((gemm_rows_kernel<TA, TW, TO, MODE>), rows_grid, dim3(256), 0, s,

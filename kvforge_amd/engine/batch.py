@@ -16,27 +16,18 @@ from typing import Sequence
 import numpy as np
 import torch
 
-ROWS_PER_TILE = 16  # rows of (query token, head in group) one prefill workgroup handles
-DECODE_KEYS_PER_SPLIT = 512
-MAX_DECODE_SPLITS = 64  # what the merge kernel takes (one lane per cut)
-COMPUTE_UNITS = 256
-DECODE_SKEW_MAX_CUTS = 8
 
 
-def skew_cuts(max_ctx: int, sum_ctx: int, n: int) -> int:
-    """Cuts of the key range that uneven contexts ask for, whatever the number of sequences: a
-    sequence's keys are walked by the waves of one workgroup per kv head and cut, so one long
-    context among short ones sets the step's time (measured at 32 sequences of 32 heads: 31
-    contexts of 600 and one of 32,768 take 153 us with one cut, 60 with eight; one of 8,192
-    takes 45 and 33).  The longest walk is brought down to about twice the mean one; a power of
-    two, so that captured launches change seldom."""
-    if n <= 1 or max_ctx < 4 * DECODE_KEYS_PER_SPLIT or sum_ctx <= 0:
-        return 1
-    want = min(max_ctx * n / (2.0 * sum_ctx), max_ctx // DECODE_KEYS_PER_SPLIT, DECODE_SKEW_MAX_CUTS)
-    cuts = 1
-    while cuts * 2 <= want:
-        cuts *= 2
-    return cuts
+@dataclass(frozen=True)
+class DecodeShape:
+    """What the single-token sequences of a step look like, as far as a part's launches may
+    depend on it besides the padded batch size: how many hold a context, the longest context
+    and the sum of all.  Parts turn it into a launch key (``Part.launch_key``); steps with equal
+    keys may replay the same captured launches."""
+
+    n: int
+    max_ctx: int
+    sum_ctx: int
 
 
 @dataclass
@@ -178,11 +169,11 @@ class Step:
         self.host_slot_ids: list[int] = []
         self.host_token_ids: np.ndarray | None = None
         self.prefill_seqs: list[int] = []
-        self.max_decode_ctx = 0
-        self.decode_skew = 1     # cuts of the key range asked for by uneven contexts (skew_cuts)
+        self.decode_shape = DecodeShape(0, 0, 0)
         self.max_position = 0
-        self._work: dict[tuple[int, int], torch.Tensor | None] = {}
-        self._identity_rotary = None
+        # What parts keep for the length of the step (work lists, launch plans, tables), under
+        # keys of their own choosing: the step knows nothing of any part's tiling.
+        self.scratch: dict = {}
         self.device: torch.device | str = "cuda"
         # A product still owed to the residual stream: (stream, product).  A part that ends in a
         # library product over many rows leaves it here instead of running an add kernel; the
@@ -210,55 +201,6 @@ class Step:
             from kvforge_amd.kernels import ops
             ops.add_rows(*self.owed)
             self.owed = None
-
-    def prefill_work(self, group_size: int, rows_per_item: int = ROWS_PER_TILE
-                     ) -> torch.Tensor | None:
-        """``[num_work, 3]`` rows (sequence row, item, item or -1) for every query run longer than
-        one token: a run of ``q`` tokens has ``q * group_size`` rows per kv head, an item covers
-        ``rows_per_item`` of them, and a workgroup takes the items of one row one after the other.
-        Item ``i`` is paired with item ``n - 1 - i``: under the causal mask the early one walks
-        few keys and the late one many, so every pair has about the same to do."""
-        if not self.prefill_seqs:
-            return None
-        key = (group_size, rows_per_item)
-        w = self._work.get(key)
-        if w is None:
-            rows = []
-            for b in self.prefill_seqs:
-                n = -(-self.q_lens[b] * group_size // rows_per_item)
-                rows += [(b, i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
-            w = torch.tensor(rows, dtype=torch.int32).reshape(-1, 3).to(self.device)
-            self._work[key] = w
-        return w
-
-    def no_rotation(self) -> tuple[torch.Tensor, torch.Tensor]:
-        """cos/sin tables of a rotation by zero, for mixers without rotary positions: one pair
-        per head is "rotated" by the identity."""
-        if self._identity_rotary is None:
-            n = int(self.positions.shape[0]) if self.positions is not None else 1
-            length = max(self.max_position + 1, n, 1)
-            self._identity_rotary = (torch.ones(length, 1, dtype=torch.float32, device=self.device),
-                                     torch.zeros(length, 1, dtype=torch.float32, device=self.device))
-        return self._identity_rotary
-
-    def decode_plan(self, H: int, KV: int, d: int, window: int):
-        """How many splits of the key range the decode kernel uses, and its workspace."""
-        G = H // KV
-        chunks = -(-G // 16)
-        ctx = min(self.max_decode_ctx, window) if window else self.max_decode_ctx
-        # Few sequences: cut the key range so that about one workgroup per compute unit pulls on
-        # the cache, each cut with at least DECODE_KEYS_PER_SPLIT keys (four key blocks for each
-        # of a workgroup's waves); below that the merge of the cuts costs more than they save.
-        # Many sequences fill the chip by themselves.
-        wgs = max(1, self.n_decode * KV * chunks)
-        splits = max(1, min(COMPUTE_UNITS // wgs, ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS))
-        # uneven contexts: the longest one is cut further, however many sequences there are
-        splits = max(splits, min(self.decode_skew, max(1, ctx // DECODE_KEYS_PER_SPLIT)))
-        if splits == 1:
-            return 1, None
-        acc = self.ws.buf("decode_part_acc", (self.n_decode * H * splits * d,), torch.float32)
-        ml = self.ws.buf("decode_part_ml", (self.n_decode * H * splits * 2,), torch.float32)
-        return splits, (acc, ml)
 
 
 def _fill_tables(meta: "MetaBuffers", host: np.ndarray, entries: Sequence[StepEntry], Bp: int,
@@ -414,9 +356,8 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
     step.host_slot_ids = slots
     step.host_token_ids = tok.copy()
     step.prefill_seqs = prefill
-    step.max_decode_ctx = int(max((ctx[b] for b in decode), default=0))
     live = [int(ctx[b]) for b in decode if ctx[b] > 0]
-    step.decode_skew = skew_cuts(step.max_decode_ctx, sum(live), len(live))
+    step.decode_shape = DecodeShape(len(live), max(live, default=0), sum(live))
     step.max_position = int(ctx.max()) if Bp else 0
-    step._work = {}
+    step.scratch = {}
     return counts

@@ -16,9 +16,8 @@ import torch
 
 from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
-from kvforge_amd.engine.batch import (DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS, MetaBuffers, Step,
-                                      StepEntry, Workspace, fill_step,
-                                      extend_tables, skew_cuts)
+from kvforge_amd.engine.batch import (DecodeShape, MetaBuffers, Step, StepEntry, Workspace,
+                                      extend_tables, fill_step)
 from kvforge_amd.kernels import ops
 from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
@@ -54,10 +53,10 @@ class ModelRunner:
         self._windowed = [g.window is not None for g in groups]
         self.num_forward_passes = 0
         self.num_tokens_processed = 0
-        # decode steps replayed from HIP graphs: (padded batch, context bucket) -> captured graph;
+        # decode steps replayed from HIP graphs: (padded batch, the parts' launch keys) -> graph;
         # only if every part's launches may be replayed for another batch
         self.use_graphs = bool(use_graphs) and all(p.replayable for p in model.spec.all_parts())
-        self.graphs: dict[tuple[int, tuple[int, int]], _DecodeGraph] = {}
+        self.graphs: dict[tuple[int, tuple], _DecodeGraph] = {}
         self.num_graph_replays = 0
         cap = self.meta.max_seqs
         # floats: temperatures, top-p, then MAX_DECODE_RUN rows of uniform numbers; ints: top-k,
@@ -213,14 +212,9 @@ class ModelRunner:
             bucket *= 2
         bucket = min(bucket, self.meta.max_seqs)
         step, _ = self.build_step(entries, pad_to=bucket, lookahead=lookahead)
-        # The longest context enters the captured launches only through the number of cuts of
-        # the key range, which grows by one per DECODE_KEYS_PER_SPLIT keys up to a limit: graphs
-        # are kept per such cell, planned for the cell's lower edge.
-        ctx_bucket = min(step.max_decode_ctx // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
-        step.max_decode_ctx = max(ctx_bucket * DECODE_KEYS_PER_SPLIT, 1)
-        # uneven contexts ask for further cuts (a power of two): a cell of its own
-        skew = skew_cuts(step.max_decode_ctx, sum(e.start_pos + 1 for e in entries), b)
-        step.decode_skew = skew
+        # The contexts' lengths enter the captured launches only through what the parts make of
+        # them (a mixer's cuts of the key range, say): graphs are kept per such key.
+        launch_key = self.model.launch_key(step.decode_shape)
         cap = self.meta.max_seqs
         fh, ih = self._sample_f_np, self._sample_i_np
         ids = [e.request_id for e in entries]
@@ -248,7 +242,7 @@ class ModelRunner:
         if dirty:
             self._sample_f.copy_(self._sample_f_host, non_blocking=True)
         self._run_counter.zero_()
-        key = (bucket, (ctx_bucket, skew))
+        key = (bucket, launch_key)
         graph = self.graphs.get(key)
         replays = k
         if graph is None:
@@ -275,9 +269,8 @@ class ModelRunner:
         starts = [p + k for p in run.begins]     # where the following run begins
         if any(s + k > self.max_model_len for s in starts):
             return None
-        ctx_bucket = min((max(starts) + 1) // DECODE_KEYS_PER_SPLIT, MAX_DECODE_SPLITS)
-        skew = skew_cuts(max(ctx_bucket * DECODE_KEYS_PER_SPLIT, 1), sum(s + 1 for s in starts), len(starts))
-        graph = self.graphs.get((run.bucket, (ctx_bucket, skew)))
+        shape = DecodeShape(len(starts), max(starts) + 1, sum(s + 1 for s in starts))
+        graph = self.graphs.get((run.bucket, self.model.launch_key(shape)))
         if graph is None:
             return None
         base = k if run.base == 0 else 0

@@ -608,9 +608,9 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
                 token_is_seq: bool = False) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
-    each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  On the
-    matrix cores the key range may be cut into ``splits`` runs; ``workspace`` then holds fp32
-    partial accumulators and fp32 (max, sum) pairs.  The vector-ALU kernel ignores ``splits``.
+    each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
+    range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
+    (``num_seqs * H * splits * d``) and fp32 (max, sum) pairs (``num_seqs * H * splits * 2``).
     ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
     single tokens), which spares the matrix-core kernel a dependent load."""
     H, KV, d = num_heads, num_kv_heads, head_dim
@@ -624,10 +624,8 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     elif num_seqs > n_seqs:
         raise KernelError("attn_decode: more sequences than block-table rows")
     nb, _, bs, _ = k_pages.shape
-    if not attention_on_matrix_cores(q.dtype, bs):
-        _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, seq_ids, num_seqs,
-                      -(-(H // KV) // 16), out, H, KV, d, scale, window, n_seqs)
-        return
+    if not 1 <= splits <= 64:
+        raise KernelError(f"attn_decode: 1 to 64 cuts of the key range, got {splits}")
     pa = pm = None
     if splits > 1:
         if workspace is None:
@@ -637,6 +635,16 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         _check(pm, "workspace[1]", F32)
         if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
             raise KernelError("attn_decode: workspace too small")
+    if not attention_on_matrix_cores(q.dtype, bs):
+        f = _fn("attn_generic", "kvf_attn_generic_decode",
+                [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+        _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+              block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
+              None if token_is_seq else cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
+              pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
+              num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
+              int(window), n_seqs, int(splits), float(scale), _stream()), "attn_generic_decode")
+        return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
             [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),

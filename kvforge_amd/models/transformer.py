@@ -9,7 +9,7 @@ import torch
 from kvforge_amd import registry
 from kvforge_amd.cache.manager import CacheGroup
 from kvforge_amd.kernels import library
-from kvforge_amd.parts.base import CacheSpec, LayerState, ModelSpec, StateSpec
+from kvforge_amd.parts.base import Block, CacheSpec, LayerState, ModelSpec, StateSpec
 from kvforge_amd.weights.loader import load_model_weights
 
 
@@ -108,6 +108,17 @@ class Transformer:
         spec = self.spec
         total = sum(p.num_bytes() for p in (spec.embedding, spec.final_norm, spec.head, *spec.positions))
         return total + sum(spec.blocks[c.layer].num_bytes() for c in self.order)
+
+    def launch_key(self, shape) -> tuple:
+        """The distinct launch keys of the model's parts for a step of single tokens (see
+        ``Part.launch_key``): what captured decode steps are kept by, beside the batch size."""
+        keys = []
+        for top in self.spec.all_parts():
+            for p in (top, *(top.parts() if isinstance(top, Block) else ())):
+                k = p.launch_key(shape)
+                if k is not None and k not in keys:
+                    keys.append(k)
+        return tuple(keys)
 
     @property
     def resident_bytes(self) -> int:

@@ -17,6 +17,57 @@ from kvforge_amd.parts.base import CacheSpec, LayerState, Mixer, WeightSpec, add
 from kvforge_amd.parts.positions import RotaryPositions
 from kvforge_amd.registry import register_mixer
 
+# Launch planning of the decode kernels.  The key range of single-token queries is cut so that
+# about one workgroup per compute unit pulls on the cache when the sequences alone do not fill
+# the chip, each cut with at least KEYS_PER_CUT keys (below that the merge of the cuts costs more
+# than they save), and further when contexts are uneven.  Everything the launches depend on
+# besides the padded batch size is the pair (context cell, cuts for uneven contexts) that
+# ``PagedAttention.launch_key`` returns, so that captured launches can be replayed for any step
+# with the same pair.
+KEYS_PER_CUT = 512
+MAX_CUTS = 64            # what the merge kernels take
+SKEW_MAX_CUTS = 8
+_compute_units: dict[int, int] = {}
+
+
+def compute_units(device) -> int:
+    """Compute units of the device the step runs on, asked of the device once."""
+    index = torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _compute_units:
+        _compute_units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _compute_units[index]
+
+
+def skew_cuts(max_ctx: int, sum_ctx: int, n: int) -> int:
+    """Cuts of the key range that uneven contexts ask for, whatever the number of sequences: a
+    sequence's keys are walked by the waves of one workgroup per kv head and cut, so one long
+    context among short ones sets the step's time (measured at 32 sequences of 32 heads: 31
+    contexts of 600 and one of 32,768 take 153 us with one cut, 60 with eight; one of 8,192
+    takes 45 and 33).  The longest walk is brought down to about twice the mean one; a power of
+    two, so that captured launches change seldom."""
+    if n <= 1 or max_ctx < 4 * KEYS_PER_CUT or sum_ctx <= 0:
+        return 1
+    want = min(max_ctx * n / (2.0 * sum_ctx), max_ctx // KEYS_PER_CUT, SKEW_MAX_CUTS)
+    cuts = 1
+    while cuts * 2 <= want:
+        cuts *= 2
+    return cuts
+
+
+def prefill_work_rows(q_lens, prefill_seqs, group_size: int, rows_per_item: int) -> list[tuple]:
+    """Rows (sequence row, item, item or -1) for every query run longer than one token: a run of
+    ``q`` tokens has ``q * group_size`` rows per kv head, an item covers ``rows_per_item`` of
+    them, and a workgroup takes the items of one row one after the other.  Item ``i`` is paired
+    with item ``n - 1 - i``: under the causal mask the early one walks few keys and the late one
+    many, so every pair has about the same to do."""
+    rows = []
+    for b in prefill_seqs:
+        n = -(-q_lens[b] * group_size // rows_per_item)
+        rows += [(b, i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
+    return rows
+
 
 @register_mixer("attention")
 class PagedAttention(Mixer):
@@ -99,6 +150,50 @@ class PagedAttention(Mixer):
     def seal(self) -> None:
         self.w_qkv, self.w_o = ops.streamed(ops.plain_of(self.w_qkv)), ops.streamed(ops.plain_of(self.w_o))
 
+    # ------------------------------------------------------------------ launch planning
+    def launch_key(self, shape) -> tuple[int, int]:
+        """(context cell, cuts for uneven contexts): all that this part's decode launches depend
+        on besides the padded batch size.  A cell is ``KEYS_PER_CUT`` keys of the longest
+        context (of the window, for a windowed layer), and the plan is made for the cell's lower
+        edge."""
+        ctx = min(shape.max_ctx, self.window) if self.window else shape.max_ctx
+        cell = min(ctx // KEYS_PER_CUT, MAX_CUTS)
+        return cell, skew_cuts(max(cell * KEYS_PER_CUT, 1), shape.sum_ctx, shape.n)
+
+    def _decode_cuts(self, step, on_matrix_cores: bool) -> int:
+        cell, skew = self.launch_key(step.decode_shape)
+        chunks = -(-(self.H // self.KV) // (16 if on_matrix_cores else 8))
+        workgroups = max(1, step.n_decode * self.KV * chunks)
+        # the vector-ALU kernel's waves take 64 keys at a time: it is worth cutting at half the
+        # keys the matrix-core kernel wants
+        finest = cell if on_matrix_cores else 2 * cell
+        cuts = max(1, min(compute_units(step.device) // workgroups, finest, MAX_CUTS))
+        return max(cuts, min(skew, max(1, cell)))
+
+    def _prefill_work(self, step, rows_per_item: int):
+        if not step.prefill_seqs:
+            return None
+        key = ("attention.prefill_work", self.H // self.KV, rows_per_item)
+        work = step.scratch.get(key)
+        if work is None:
+            rows = prefill_work_rows(step.q_lens, step.prefill_seqs, self.H // self.KV, rows_per_item)
+            work = torch.tensor(rows, dtype=torch.int32).reshape(-1, 3).to(step.device)
+            step.scratch[key] = work
+        return work
+
+    @staticmethod
+    def _no_rotation(step) -> tuple[torch.Tensor, torch.Tensor]:
+        """cos/sin tables of a rotation by zero, for attention without rotary positions: one
+        pair per head is "rotated" by the identity."""
+        tables = step.scratch.get("attention.no_rotation")
+        if tables is None:
+            n = int(step.positions.shape[0]) if step.positions is not None else 1
+            length = max(step.max_position + 1, n, 1)
+            tables = (torch.ones(length, 1, dtype=torch.float32, device=step.device),
+                      torch.zeros(length, 1, dtype=torch.float32, device=step.device))
+            step.scratch["attention.no_rotation"] = tables
+        return tables
+
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""
         n = x.shape[0]
@@ -106,7 +201,7 @@ class PagedAttention(Mixer):
         ws = step.ws
         act = step.act_dtype
         table = step.block_tables[layer.group]
-        cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else step.no_rotation()
+        cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else self._no_rotation(step)
         rms = self.norm_eps
         owed = None
         if rms is not None and not ops.bf16_kernel_takes(x, self.w_qkv, True):
@@ -140,12 +235,16 @@ class PagedAttention(Mixer):
         out = ws.buf("attn_out", (n, H * d), act)
         window = self.window or 0
         bs = layer.k_pages.shape[2]
-        work = step.prefill_work(H // KV, ops.prefill_rows_per_item(act, d, bs))
+        work = self._prefill_work(step, ops.prefill_rows_per_item(act, d, bs))
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window)
         if step.n_decode:
-            splits, workspace = step.decode_plan(H, KV, d, window)
+            splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
+            workspace = None
+            if splits > 1:
+                workspace = (ws.buf("decode_part_acc", (step.n_decode * H * splits * d,), torch.float32),
+                             ws.buf("decode_part_ml", (step.n_decode * H * splits * 2,), torch.float32))
             ops.attn_decode(qkv, layer.k_pages, layer.v_pages, table, step.decode_seq_ids,
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,

@@ -93,6 +93,13 @@ class Part:
         (what the weights occupy, as opposed to what a step reads)."""
         return []
 
+    def launch_key(self, shape):
+        """What this part's launches for a step of single tokens depend on besides the padded
+        batch size, worked out from ``shape`` (``n`` sequences with a context, ``max_ctx``,
+        ``sum_ctx``): any hashable value.  Captured launches are replayed only for steps whose
+        parts all give the keys they were captured with.  ``None``: nothing (the default)."""
+        return None
+
     def seal(self) -> None:
         """Called once after ``load`` (and any ``absorb_norm``), before the first forward: the
         place for the last re-layout of weights, such as tiles for the weight-streaming kernel."""

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from kvforge_amd.cache import CacheGroup, CacheManager
-from kvforge_amd.engine.batch import (MetaBuffers, Step, StepEntry, Workspace, extend_tables,
+from kvforge_amd.engine.batch import (DecodeShape, MetaBuffers, Step, StepEntry, Workspace, extend_tables,
                                       fill_step)
 
 
@@ -41,9 +41,13 @@ def test_flat_varlen_batch_reference_vector():
         slot = int(step.block_tables[0][s, p // 4]) * 4 + p % 4
         assert slot == cache.slot("ab"[s], p)
     assert step.n_decode == 1 and step.decode_seq_ids.tolist() == [1] and step.prefill_seqs == [0]
-    # 3 tokens x group size over 16-row items: one item, then two paired into one row
-    assert step.prefill_work(2).tolist() == [[0, 0, -1]] and step.prefill_work(6).tolist() == [[0, 0, 1]]
-    assert step.prefill_work(6, 4).tolist() == [[0, 0, 4], [0, 1, 3], [0, 2, -1]]
+    assert step.decode_shape == DecodeShape(n=1, max_ctx=2, sum_ctx=2)
+    # attention's work list for the run of 3 tokens: 3 tokens x group size over 16-row items is
+    # one item, then two paired into one row
+    from kvforge_amd.parts.attention import prefill_work_rows
+    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 2, 16) == [(0, 0, -1)]
+    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 16) == [(0, 0, 1)]
+    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 4) == [(0, 0, 4), (0, 1, 3), (0, 2, -1)]
 
 
 def test_wanted_places_and_modes():
@@ -71,7 +75,7 @@ def test_pure_decode_padding_is_inert():
     assert step.ctx_lens.tolist() == [5, 5, 0, 0]
     assert (step.block_tables[0][2:] == -1).all()
     # a padded batch has a fixed shape: one logits row per sequence, padding included
-    assert step.max_decode_ctx == 5 and step.n_logits == 4
+    assert step.decode_shape == DecodeShape(n=2, max_ctx=5, sum_ctx=10) and step.n_logits == 4
     assert step.logits_rows.tolist() == [0, 1, 2, 3]
     with pytest.raises(ValueError, match="padding"):
         fill_step(step, meta, [StepEntry("a", [3], 4, "none")], cache.block_table, lambda r: -1, 4,
@@ -162,7 +166,7 @@ def test_workspace_hands_out_the_same_memory_until_it_grows():
 
 
 def test_uneven_contexts_ask_for_cuts_of_the_key_range():
-    from kvforge_amd.engine.batch import skew_cuts
+    from kvforge_amd.parts.attention import PagedAttention, skew_cuts
     assert skew_cuts(600, 32 * 600, 32) == 1                     # even contexts: none
     assert skew_cuts(1800, 1800 + 31 * 100, 32) == 1             # too short to be worth a merge
     assert skew_cuts(32768, 32768 + 31 * 600, 32) == 8           # one long context among short ones
@@ -172,3 +176,11 @@ def test_uneven_contexts_ask_for_cuts_of_the_key_range():
     assert skew_cuts(3000, 3000 + 3000, 2) == 1                  # twice the mean is the aim
     assert skew_cuts(2100, 2100 + 63 * 10, 64) == 4              # never cuts below 512 keys
     assert skew_cuts(40000, 40000, 1) == 1                       # one sequence: the other rule's case
+    # what a captured decode step is kept by: the cell of 512 keys the longest context (or the
+    # window) lies in, and the cuts that uneven contexts ask for at the cell's lower edge
+    full = PagedAttention("a", 64, 4, 2, 16, None)
+    windowed = PagedAttention("a", 64, 4, 2, 16, None, window=600)
+    assert full.launch_key(DecodeShape(8, 640, 8 * 600)) == (1, 1)
+    assert full.launch_key(DecodeShape(8, 511, 8 * 500)) == (0, 1)
+    assert full.launch_key(DecodeShape(32, 32768, 32768 + 31 * 600)) == (64, 8)
+    assert windowed.launch_key(DecodeShape(32, 32768, 32768 + 31 * 600)) == (1, 1)

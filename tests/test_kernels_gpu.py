@@ -424,15 +424,46 @@ def test_gemm_bf16_rows_do_not_depend_on_neighbours():
 
 
 def test_gemm_rows_do_not_depend_on_batch():
-    """fp32 products are accumulated in one fixed order: a row alone equals the row in a batch."""
+    """fp32 products are summed in a fixed order: a row alone has the bits of the row in any
+    batch that the same kernel takes (up to 32 rows: the weight-streaming one, whatever the
+    number of rows per workgroup; more: the tiled one), and the two kernels agree to rounding."""
     g = torch.Generator().manual_seed(3)
     a = torch.randn(77, 176, generator=g).to(DEV)
     w = torch.randn(300, 176, generator=g).to(DEV)
-    full = torch.empty(77, 300, device=DEV)
-    ops().gemm(a, w, full)
-    one = torch.empty(1, 300, device=DEV)
-    ops().gemm(a[40:41], w, one)
-    assert torch.equal(one[0], full[40])
+
+    def product(rows):
+        out = torch.empty(rows.shape[0], 300, device=DEV)
+        ops().gemm(rows, w, out)
+        return out
+
+    full = product(a)
+    alone = product(a[40:41])
+    for lo, hi in ((40, 42), (38, 42), (35, 43), (30, 46), (20, 52)):     # 2, 4, 8, 16, 32 rows
+        assert torch.equal(product(a[lo:hi])[40 - lo], alone[0]), (lo, hi)
+    assert torch.equal(product(a[8:77])[32], full[40])                      # 69 rows and 77
+    torch.testing.assert_close(alone[0], full[40], atol=2e-5, rtol=1e-5)
+    want = a.double() @ w.double().T
+    torch.testing.assert_close(full.double(), want, atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(alone[0].double(), want[40], atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 13, 32])
+@pytest.mark.parametrize("tw", DTYPES)
+def test_gemm_generic_few_rows_over_long_and_uneven_k(m, tw):
+    """The weight-streaming fp32 kernel: K beyond one staged chunk and not a multiple of the 256
+    elements a wave reads at a time, N that ends inside a workgroup's columns, accumulation
+    into the stream, and a row stride wider than K."""
+    g = torch.Generator().manual_seed(m)
+    n, k = 70, 2348
+    a = torch.randn(m, k + 8, generator=g).to(DEV)[:, :k]
+    w = (torch.randn(n, k, generator=g) * 0.05).to(tw).to(DEV)
+    want = a.double() @ w.double().T
+    out = torch.full((m, n), 7.0, device=DEV)
+    ops().gemm(a, w, out)
+    torch.testing.assert_close(out.double(), want, atol=3e-5, rtol=1e-5)
+    acc = torch.ones(m, n, device=DEV)
+    ops().gemm(a, w, acc, accumulate=True)
+    torch.testing.assert_close(acc.double(), want + 1.0, atol=3e-5, rtol=1e-5)
 
 
 class Paged:
@@ -525,7 +556,8 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
                                         (4, 4, 80, 16), (32, 8, 64, 16), (8, 2, 128, 16),
-                                        (12, 1, 112, 16), (2, 1, 256, 32), (20, 1, 16, 8)])
+                                        (12, 1, 112, 16), (2, 1, 256, 32), (20, 1, 16, 8),
+                                        (4, 2, 32, 6)])
 @pytest.mark.parametrize("splits", [1, 3, 7])
 @pytest.mark.parametrize("window", [0, 11])
 def test_attn_decode(dtype, H, KV, d, bs, splits, window):
