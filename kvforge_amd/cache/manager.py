@@ -21,11 +21,12 @@ RELEASED = -1  # table entry of a page that was given back (or never held)
 @dataclass(frozen=True)
 class CacheGroup:
     """Layers whose mixers have equal cache needs.  ``layers``: places in the model's run order
-    of the calls that own pages in this group."""
+    of the calls that own pages in this group; ``pages``: the tensors a page consists of, as
+    the mixers declare them (``parts.base.PageTensor``; the manager itself only counts pages
+    and never looks at them)."""
 
     layers: tuple[int, ...]
-    num_kv_heads: int
-    head_dim: int
+    pages: tuple = ()
     window: int | None = None
 
 

@@ -1,10 +1,10 @@
-"""Device storage behind the cache manager: K and V pages per cache-owning call, and state
-tensors ``[num_slots, *shape]`` for mixers with fixed-size state.  K pages are
-``[num_blocks, kv_heads, block_size, head_dim]`` (one (page, head) tile is contiguous, a key's
-elements side by side); V pages are transposed, ``[num_blocks, kv_heads, head_dim, block_size]``
-(an element's keys side by side), which is the order the matrix cores contract ``P * V`` in.
-The reference keeps ``[num_blocks, block_size, kv_heads, head_dim]`` for both
-(src/tokenvault/cache/kv_cache.py:27-31).
+"""Device storage behind the cache manager: for every cache-owning call the page tensors its
+mixer declares (``CacheSpec.pages``), each ``[num_blocks, *page shape]``, and state tensors
+``[num_slots, *shape]`` for mixers with fixed-size state.  Attention declares K pages
+``[kv_heads, block_size, head_dim]`` (one (page, head) tile is contiguous, a key's elements side
+by side) and V pages transposed, ``[kv_heads, head_dim, block_size]`` (an element's keys side by
+side), which is the order the matrix cores contract ``P * V`` in.  The reference keeps
+``[num_blocks, block_size, kv_heads, head_dim]`` for both (src/tokenvault/cache/kv_cache.py:27-31).
 """
 
 from __future__ import annotations
@@ -19,20 +19,18 @@ class PagedStorage:
     def __init__(self, groups: list[CacheGroup], num_blocks: list[int], block_size: int,
                  dtype: torch.dtype, device: torch.device | str) -> None:
         self.block_size, self.dtype = block_size, dtype
-        self.k: dict[int, torch.Tensor] = {}
-        self.v: dict[int, torch.Tensor] = {}
+        self.pages: dict[int, dict[str, torch.Tensor]] = {}    # owning call -> name -> tensor
         self.group_of: dict[int, int] = {}
         for g, (grp, nb) in enumerate(zip(groups, num_blocks)):
-            k_shape = (nb, grp.num_kv_heads, block_size, grp.head_dim)
-            v_shape = (nb, grp.num_kv_heads, grp.head_dim, block_size)
             for layer in grp.layers:
-                self.k[layer] = torch.zeros(k_shape, dtype=dtype, device=device)
-                self.v[layer] = torch.zeros(v_shape, dtype=dtype, device=device)
+                self.pages[layer] = {
+                    t.name: torch.zeros((nb, *t.page_shape(block_size)), dtype=t.dtype or dtype,
+                                        device=device) for t in grp.pages}
                 self.group_of[layer] = g
 
     @property
     def memory_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in list(self.k.values()) + list(self.v.values()))
+        return sum(t.numel() * t.element_size() for held in self.pages.values() for t in held.values())
 
 
 class StateStorage:
@@ -43,6 +41,7 @@ class StateStorage:
 
 
 def bytes_per_block(groups: list[CacheGroup], block_size: int, dtype: torch.dtype) -> int:
-    """K and V of one page over every layer of every group (src/tokenvault/config.py:91-95)."""
-    elem = torch.tensor([], dtype=dtype).element_size()
-    return sum(2 * len(g.layers) * block_size * g.num_kv_heads * g.head_dim * elem for g in groups)
+    """What one page number costs over every layer of every group: for attention K and V,
+    ``2 * layers * block_size * kv_heads * head_dim * element size``
+    (src/tokenvault/config.py:91-95)."""
+    return sum(len(g.layers) * sum(t.page_bytes(block_size, dtype) for t in g.pages) for g in groups)

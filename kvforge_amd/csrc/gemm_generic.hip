@@ -146,7 +146,6 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A
 }
 
 // ---- few rows, W streamed once: see the head of the file.
-constexpr int SW = 4;        // waves per workgroup
 constexpr int SKC = 1024;    // elements of K per staged chunk of A
 constexpr int SQ = 4 * KVF_WAVE;  // elements of K a wave reads per step (16 bytes a lane)
 
@@ -165,9 +164,12 @@ template <> struct Quad<bf16_t> {
 // MT rows per workgroup (1, 2, 4, 8 or 16); SN columns of W per wave, each read DEPTH steps
 // ahead, so that SN * DEPTH loads of 16 bytes are in flight per lane: narrow outputs (few
 // columns, hence few waves) take one column per wave and look far ahead, wide ones four columns.
-// The sums do not depend on MT, SN or DEPTH.  Needs K % 4 == 0 and rows of A and W that start on
+// SW waves per workgroup share the staged rows of A: with one column per wave a workgroup of four
+// waves would stage all of A for four columns of W and move twice the bytes of W through LDS,
+// so narrow outputs get sixteen waves per workgroup.
+// The sums do not depend on MT, SN, DEPTH or SW.  Needs K % 4 == 0 and rows of A and W that start on
 // 16 bytes (8 for bf16): the caller checks.
-template <typename TA, typename TW, typename TO, int MODE, int MT, int SN, int DEPTH>
+template <typename TA, typename TW, typename TO, int MODE, int MT, int SN, int DEPTH, int SW>
 __global__ __launch_bounds__(SW * KVF_WAVE) void gemm_stream_kernel(
     const TA* __restrict__ A, const TW* __restrict__ W, TO* __restrict__ C, int M, int N, int K,
     int lda, int ldc) {
@@ -247,16 +249,16 @@ __global__ __launch_bounds__(SW * KVF_WAVE) void gemm_stream_kernel(
 
 template <typename TA, typename TW, typename TO, int MODE, int MT>
 int launch_stream(const TA* A, const TW* W, TO* C, int M, int N, int K, int lda, int ldc, hipStream_t s) {
-#define GO(SN, DEPTH)                                                                            \
+#define GO(SN, DEPTH, SW)                                                                        \
   do {                                                                                           \
     dim3 grid((N + SN * SW - 1) / (SN * SW), (M + MT - 1) / MT);                                 \
-    hipLaunchKernelGGL((gemm_stream_kernel<TA, TW, TO, MODE, MT, SN, DEPTH>), grid,              \
+    hipLaunchKernelGGL((gemm_stream_kernel<TA, TW, TO, MODE, MT, SN, DEPTH, SW>), grid,          \
                        dim3(SW * KVF_WAVE), 0, s, A, W, C, M, N, K, lda, ldc);                   \
   } while (0)
   // about four waves or more per compute unit's SIMD at the widest choice that allows it
-  if (N >= 16384) GO(4, 2);
-  else if (N >= 6144) GO(2, 4);
-  else GO(1, 8);
+  if (N >= 16384) GO(4, 2, 4);
+  else if (N >= 6144) GO(2, 4, 8);
+  else GO(1, 8, 16);
 #undef GO
   return kvf_last_error();
 }

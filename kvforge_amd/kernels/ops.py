@@ -2,7 +2,10 @@
 devices and strides are what its kernel and launch grid assume, then launches on torch's
 current stream (so launches made while a torch HIP-graph capture is active are captured).
 
-There is no fallback: every function here runs a hand-written gfx950 kernel or raises.
+There is no fallback: every function here runs a hand-written gfx950 kernel, or (``gemm`` for
+bf16 with many rows, as the reference's engine does for its products) the library's matrix
+product through ``csrc/gemm_library.hip``, or raises.  No torch operator computes anything
+here.
 """
 
 from __future__ import annotations
@@ -339,35 +342,43 @@ def k_halves_pay(a: torch.Tensor, w) -> bool:
 
 # The library's product is called through an entry point of our own: torch.mm costs 17 us of
 # host time a call, which is what bounds a step that is launched kernel by kernel (a portion of a
-# prompt) at a few hundred rows.  LIBRARY_DIRECT = False sends them through torch.mm again.
-LIBRARY_DIRECT = True
+# prompt) at a few hundred rows.
 LIBRARY_WORKSPACE_BYTES = 76 << 20
 _library_ready: dict[int, bool] = {}
 _LIBRARY_ARGS = [c_void_p, c_void_p, c_void_p] + [c_int] * 7 + [c_void_p]
 
 
-def _library_product(a, w, out, accumulate, m, n, k, lda, ldc) -> bool:
+def library_ready(device) -> None:
+    """Set the library product up on ``device`` (its workspace is allocated here, once): to be
+    called outside any stream capture, which ``gemm`` does by itself on its first library
+    product."""
+    dev = torch.device(device).index
+    if dev is None:
+        dev = torch.cuda.current_device()
+    if _library_ready.get(dev):
+        return
+    if torch.cuda.is_current_stream_capturing():
+        raise KernelError("the library product has to be set up before a stream is captured: "
+                          "run the step once (or call ops.library_ready) outside the capture")
+    init = _fn("gemm_library", "kvf_gemm_library_init", [c_long])
+    with torch.cuda.device(dev):
+        _ok(init(LIBRARY_WORKSPACE_BYTES), "gemm_library_init")
+    _library_ready[dev] = True
+
+
+def _library_product(a, w, out, accumulate, m, n, k, lda, ldc) -> None:
     """``out = a @ w.T`` (or ``+=``, in fp32) by hipBLASLt, with fp32 sums stored as ``out`` has
-    them.  False where that route is closed: switched off, not set up yet while a stream is
-    being captured (its workspace cannot be allocated then), or no algorithm for the shape."""
-    if not LIBRARY_DIRECT or out.dtype not in (F32, BF16) or (accumulate and out.dtype != F32):
-        return False
-    dev = a.device.index if a.device.index is not None else torch.cuda.current_device()
-    ready = _library_ready.get(dev)
-    if ready is None:
-        if torch.cuda.is_current_stream_capturing():
-            return False
-        init = _fn("gemm_library", "kvf_gemm_library_init", [c_long])
-        with torch.cuda.device(dev):
-            _ok(init(LIBRARY_WORKSPACE_BYTES), "gemm_library_init")
-        ready = _library_ready[dev] = True
+    them.  Raises where the library names no algorithm for the shape."""
+    if out.dtype not in (F32, BF16) or (accumulate and out.dtype != F32):
+        raise KernelError(f"library product: output must be float32 or bfloat16, got {out.dtype}")
+    library_ready(a.device)
     f = _fn("gemm_library", "kvf_gemm_library_bf16", _LIBRARY_ARGS)
     code = f(a.data_ptr(), w.data_ptr(), out.data_ptr(), 1 if out.dtype == F32 else 0,
              1 if accumulate else 0, m, n, k, lda, ldc, _stream())
     if code == -1:
-        return False
+        raise KernelError(f"the library has no bf16 product for {m} x {n} x {k} "
+                          f"(row strides {lda} / {ldc})")
     _ok(code, "gemm_library")
-    return True
 
 
 def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
@@ -414,19 +425,11 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
                   half_out.data_ptr() if half_out is not None else None, _stream()), "gemm_bf16")
             return
         if owed is not None:
-            out.add_(owed)
-        if _library_product(a, plain_of(w), out, accumulate, m, n, k, lda, ldc):
-            return
-        if accumulate:
-            # many rows: the library's bf16 product, then the residual sum in fp32
-            out.add_(torch.mm(a, plain_of(w).t()))
-        elif out.dtype == F32:
-            out.copy_(torch.mm(a, plain_of(w).t()))
-        else:
-            torch.mm(a, plain_of(w).t(), out=out)
+            add_rows(out, owed)
+        _library_product(a, plain_of(w), out, accumulate, m, n, k, lda, ldc)
         return
     if owed is not None:
-        out.add_(owed)
+        add_rows(out, owed)
     w = plain_of(w)
     f = _fn("gemm_generic", "kvf_gemm_generic",
             [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6 + [c_void_p])

@@ -40,7 +40,7 @@ class Transformer:
         by_spec: dict[CacheSpec, list[int]] = {}
         for i in owners:
             by_spec.setdefault(spec.blocks[self.order[i].layer].mixer.cache_spec, []).append(i)
-        self.cache_groups = [CacheGroup(tuple(ix), cs.num_kv_heads, cs.head_dim, cs.window)
+        self.cache_groups = [CacheGroup(tuple(ix), cs.pages, cs.window)
                              for cs, ix in by_spec.items()]
         self.state_specs: dict[int, StateSpec] = {
             i: spec.blocks[c.layer].mixer.state_spec for i, c in enumerate(self.order)
@@ -94,8 +94,8 @@ class Transformer:
         for i, c in enumerate(self.order):
             src = i if c.cache_of is None else c.cache_of
             ls = LayerState(owns_cache=c.cache_of is None)
-            if src in storage.k:
-                ls.group, ls.k_pages, ls.v_pages = storage.group_of[src], storage.k[src], storage.v[src]
+            if src in storage.pages:
+                ls.group, ls.pages = storage.group_of[src], storage.pages[src]
             if states is not None and i in states.tensors:
                 ls.state = states.tensors[i]
             self.layer_states.append(ls)

@@ -13,7 +13,8 @@ import math
 import torch
 
 from kvforge_amd.kernels import ops
-from kvforge_amd.parts.base import CacheSpec, LayerState, Mixer, WeightSpec, add_product
+from kvforge_amd.parts.base import (CacheSpec, LayerState, Mixer, WeightSpec, add_product,
+                                    attention_pages)
 from kvforge_amd.parts.positions import RotaryPositions
 from kvforge_amd.registry import register_mixer
 
@@ -89,7 +90,7 @@ class PagedAttention(Mixer):
         self.rotary = rotary
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         self.window = int(window) if window else None
-        self.cache_spec = CacheSpec(self.KV, self.d, self.window)
+        self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
 

@@ -31,16 +31,49 @@ class WeightSpec:
     integer: bool = False
 
 
+BLOCK = "block"   # stands for the page size (tokens per page) in a ``PageTensor``'s shape
+
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor of a mixer's pages: ``name`` is what the mixer finds it under in
+    ``LayerState.pages``, ``shape`` the shape of one page, in which ``BLOCK`` stands for the
+    number of tokens a page holds (so the mixer chooses where the token index lies), ``dtype``
+    the element type (``None``: the engine's)."""
+
+    name: str
+    shape: tuple
+    dtype: torch.dtype | None = None
+
+    def page_shape(self, block_size: int) -> tuple[int, ...]:
+        return tuple(block_size if s == BLOCK else int(s) for s in self.shape)
+
+    def page_bytes(self, block_size: int, engine_dtype: torch.dtype) -> int:
+        n = 1
+        for s in self.page_shape(block_size):
+            n *= s
+        return n * torch.tensor([], dtype=self.dtype or engine_dtype).element_size()
+
+
+def attention_pages(num_kv_heads: int, head_dim: int) -> tuple[PageTensor, PageTensor]:
+    """Keys ``[kv heads, block, head size]`` (a key's elements side by side) and values
+    transposed, ``[kv heads, head size, block]`` (an element's keys side by side, the order in
+    which the matrix cores contract ``P * V``)."""
+    return (PageTensor("k", (num_kv_heads, BLOCK, head_dim)),
+            PageTensor("v", (num_kv_heads, head_dim, BLOCK)))
+
+
 @dataclass(frozen=True)
 class CacheSpec:
-    """A mixer's need for keys and values that grow with the sequence.
+    """A mixer's need for per-token memory that grows with the sequence: the tensors its pages
+    consist of (keys and values for attention; any others for another mixer, one latent vector
+    per token, say).
 
     ``window``: ``None`` keeps every position; ``w`` keeps the last ``w`` positions, and pages
     wholly behind the window are given back while the request is live.  Layers with equal specs
     form one cache group with pages and block tables of its own."""
 
-    num_kv_heads: int
-    head_dim: int
+    pages: tuple[PageTensor, ...]
     window: int | None = None
 
 
@@ -58,10 +91,17 @@ class LayerState:
     (possibly another block's), the group whose block tables address them, and its state slots."""
 
     group: int | None = None
-    k_pages: torch.Tensor | None = None
-    v_pages: torch.Tensor | None = None
+    pages: dict[str, torch.Tensor] = field(default_factory=dict)   # by ``PageTensor.name``
     owns_cache: bool = True
     state: torch.Tensor | None = None
+
+    @property
+    def k_pages(self) -> torch.Tensor | None:
+        return self.pages.get("k")
+
+    @property
+    def v_pages(self) -> torch.Tensor | None:
+        return self.pages.get("v")
 
 
 class Part:

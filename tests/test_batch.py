@@ -12,7 +12,7 @@ from kvforge_amd.engine.batch import (DecodeShape, MetaBuffers, Step, StepEntry,
 
 
 def setup(num_blocks=16, bs=4, groups=None):
-    groups = groups or [CacheGroup((0,), 1, 16, None)]
+    groups = groups or [CacheGroup((0,))]
     cache = CacheManager(bs, groups, num_blocks)
     meta = MetaBuffers(64, 8, [8] * len(groups), "cpu")
     step = Step()

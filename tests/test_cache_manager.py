@@ -8,10 +8,12 @@ import random
 
 import pytest
 
+from kvforge_amd.parts import attention_pages
+
 from kvforge_amd.cache import (RELEASED, BlockPool, CacheGroup, CacheManager, NoFreeBlocksError,
                                StateSlots)
 
-FULL = CacheGroup(layers=(0, 1), num_kv_heads=2, head_dim=16, window=None)
+FULL = CacheGroup(layers=(0, 1), pages=attention_pages(2, 16), window=None)
 
 
 def mgr(num_blocks, block_size, groups=(FULL,), **kw):
@@ -97,8 +99,8 @@ def test_lifo_reuse():
 
 
 def test_window_group_gives_pages_back_early():
-    win = CacheGroup(layers=(1,), num_kv_heads=1, head_dim=16, window=6)
-    m = mgr(8, 4, groups=(CacheGroup((0,), 1, 16, None), win))
+    win = CacheGroup(layers=(1,), pages=attention_pages(1, 16), window=6)
+    m = mgr(8, 4, groups=(CacheGroup((0,), attention_pages(1, 16), None), win))
     m.allocate("a", 0)
     m.append_slots("a", 10, 0)
     assert len(m.block_table("a", 0)) == 3 and len(m.block_table("a", 1)) == 3
@@ -116,7 +118,7 @@ def test_window_group_gives_pages_back_early():
 
 
 def test_window_group_needs_fewer_pages_for_later_portions():
-    win = CacheGroup(layers=(0,), num_kv_heads=1, head_dim=16, window=4)
+    win = CacheGroup(layers=(0,), pages=attention_pages(1, 16), window=4)
     m = mgr(3, 4, groups=(win,))
     m.allocate("a", 0)
     m.append_slots("a", 8, 0)                      # two pages
@@ -150,7 +152,8 @@ def test_random_orders_lose_nothing(seed):
     held by exactly one table entry, counts agree, and at the end everything is free."""
     rng = random.Random(seed)
     bs = rng.choice([4, 8, 16])
-    groups = (CacheGroup((0, 2), 2, 16, None), CacheGroup((1,), 1, 32, rng.choice([5, 16, 40])))
+    groups = (CacheGroup((0, 2), attention_pages(2, 16), None),
+              CacheGroup((1,), attention_pages(1, 32), rng.choice([5, 16, 40])))
     counts = [rng.randint(8, 24), rng.randint(8, 24)]
     m = CacheManager(bs, list(groups), counts, num_state_slots=5)
     live: dict[str, int] = {}

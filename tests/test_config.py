@@ -108,3 +108,18 @@ def test_model_spec_has_no_size_of_its_own():
         assert len([k for k in shapes if k.endswith("input_layernorm.weight")]) == d["num_hidden_layers"]
         blk = spec.blocks[0]
         assert blk.mixer_norm.eps == d["rms_norm_eps"] and blk.mixer.scale == pytest.approx(hd ** -0.5)
+
+
+def test_bytes_per_block_follow_from_the_page_tensors_the_mixers_declare():
+    """Llama 3.2 1B in bf16 with pages of 16 tokens: 2 * 16 layers * 16 * 8 heads * 64 * 2 bytes
+    (src/tokenvault/config.py:91-95), worked out from what attention declares as its pages."""
+    import torch
+    from kvforge_amd import registry
+    from kvforge_amd.cache.storage import bytes_per_block
+    from kvforge_amd.models.transformer import Transformer
+    model = Transformer(registry.build_spec(registry.config_from_dict(preset_dict("llama-1b"))),
+                        torch.bfloat16, "cpu")
+    assert [len(g.layers) for g in model.cache_groups] == [16]
+    assert [t.name for t in model.cache_groups[0].pages] == ["k", "v"]
+    assert bytes_per_block(model.cache_groups, 16, torch.bfloat16) == 524288
+    assert bytes_per_block(model.cache_groups, 16, torch.float32) == 2 * 524288

@@ -15,6 +15,7 @@ import torch
 import kvforge_amd
 from kvforge_amd import registry
 from kvforge_amd.cache import CacheGroup, CacheManager
+from kvforge_amd.parts import attention_pages
 from kvforge_amd.config.model import ModelConfig
 from kvforge_amd.engine.batch import MetaBuffers, Step, StepEntry, Workspace, fill_step
 from kvforge_amd.engine.runner import ModelRunner
@@ -125,10 +126,10 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
          "a.o_proj.weight": rand(hidden, H * d, seed=13, scale=0.1).to(dtype)}
     part.load({k: v.to(DEV) for k, v in w.items()})
     part.seal()
-    cache = CacheManager(bs, [CacheGroup((0,), KV, d, window)], 24)
+    cache = CacheManager(bs, [CacheGroup((0,), attention_pages(KV, d), window)], 24)
     ls = LayerState(group=0, owns_cache=True,
-                    k_pages=torch.zeros(24, KV, bs, d, dtype=dtype, device=DEV),
-                    v_pages=torch.zeros(24, KV, d, bs, dtype=dtype, device=DEV))
+                    pages={"k": torch.zeros(24, KV, bs, d, dtype=dtype, device=DEV),
+                           "v": torch.zeros(24, KV, d, bs, dtype=dtype, device=DEV)})
     xs = {"s": rand(21, hidden, seed=14).to(dtype), "t": rand(9, hidden, seed=15).to(dtype)}
     cfg = {"num_attention_heads": H, "num_key_value_heads": KV, "head_dim": d}
     want = {}
@@ -175,10 +176,11 @@ def test_pre_norm_block(dtype, n):
     block.load({k: v.to(DEV) for k, v in w.items()})
     block.seal()
     x = rand(n, hidden, seed=21)
-    cache = CacheManager(4, [CacheGroup((0,), KV, d, None)], 8)
+    cache = CacheManager(4, [CacheGroup((0,), attention_pages(KV, d), None)], 8)
     cache.allocate("r", n)
-    ls = LayerState(group=0, owns_cache=True, k_pages=torch.zeros(8, KV, 4, d, dtype=dtype, device=DEV),
-                    v_pages=torch.zeros(8, KV, d, 4, dtype=dtype, device=DEV))
+    ls = LayerState(group=0, owns_cache=True,
+                    pages={"k": torch.zeros(8, KV, 4, d, dtype=dtype, device=DEV),
+                           "v": torch.zeros(8, KV, d, 4, dtype=dtype, device=DEV)})
     step = make_step([StepEntry("r", [0] * n, 0, "none")], cache, dtype)
     residual = x.clone().to(DEV)
     block.forward(residual, step, ls)

@@ -18,7 +18,7 @@ from kvforge_amd.sampling import SamplingParams
 class Driver:
     def __init__(self, num_blocks=64, block_size=4, run_steps=1, run_ahead=False, device_runs=None,
                  **limits):
-        cache = CacheManager(block_size, [CacheGroup((0,), 1, 16, None)], num_blocks)
+        cache = CacheManager(block_size, [CacheGroup((0,))], num_blocks)
         self.sched = Scheduler(SchedulerConfig(**limits), cache, run_steps, run_ahead,
                                device_runs=device_runs)
         self.cache = cache
@@ -182,7 +182,7 @@ def test_the_head_of_the_line_is_not_overtaken():
 
 
 def test_the_watermark_keeps_nobody_out_of_an_empty_pool():
-    cache = CacheManager(4, [CacheGroup((0,), 1, 16, None)], 8, watermark=0.25)
+    cache = CacheManager(4, [CacheGroup((0,))], 8, watermark=0.25)
     sched = Scheduler(SchedulerConfig(), cache)
     sched.add_request(Request("fills", range(30), SamplingParams(max_tokens=2), arrival_time=0.0))
     sched.add_request(Request("next", range(4), SamplingParams(max_tokens=2), arrival_time=1.0))

@@ -1,0 +1,196 @@
+"""A mixer whose growing memory is not keys and values: one latent vector per token, kept in a
+single page tensor of its own shape and element type, declared through ``CacheSpec.pages``.  It is
+defined here with torch ops, registered beside the built-in attention in a toy architecture (so
+the model has two cache groups with pages of different make), stepped in portions with pages
+that are used again, and compared with the same model written out over whole sequences.  Nothing
+in the framework's files knows of it."""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Any
+
+import pytest
+import torch
+
+import kvforge_amd
+from kvforge_amd.cache.storage import bytes_per_block
+from kvforge_amd.config.model import ModelConfig
+from kvforge_amd.engine.batch import StepEntry
+from kvforge_amd.engine.runner import ModelRunner
+from kvforge_amd.models.transformer import Transformer
+from kvforge_amd.parts import (BLOCK, CacheSpec, LMHead, Mixer, ModelSpec, PagedAttention, PageTensor,
+                               PreNormBlock, RMSNorm, RotaryPositions, SwiGLU, TokenEmbedding,
+                               WeightSpec)
+from tests.plain import llama as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+class ToyLatentMixer(Mixer):
+    """``c_t = x_t Wc^T`` (``rank`` numbers) is all that is remembered of token ``t``; a query
+    ``q_t = x_t Wq^T`` weighs the latents at or before it by ``softmax(q_t . c_j / sqrt(rank))``
+    and the mix goes through ``Wo``.  Pages: one tensor ``latent [block, rank]`` in fp32 whatever
+    the engine's type."""
+
+    def __init__(self, prefix: str, hidden: int, rank: int) -> None:
+        self.prefix, self.hidden, self.rank = prefix, hidden, rank
+        self.cache_spec = CacheSpec((PageTensor("latent", (BLOCK, rank), torch.float32),))
+
+    def weight_specs(self):
+        return {self._name("c.weight"): WeightSpec((self.rank, self.hidden), std=0.3),
+                self._name("q.weight"): WeightSpec((self.rank, self.hidden), std=0.3),
+                self._name("o.weight"): WeightSpec((self.hidden, self.rank), std=0.3)}
+
+    def load(self, tensors):
+        self.wc, self.wq, self.wo = (tensors[self._name(f"{n}.weight")].float() for n in "cqo")
+
+    def forward(self, x, step, layer, residual):
+        pages = layer.pages["latent"]                       # [num_blocks, block, rank]
+        bs = pages.shape[1]
+        table = step.block_tables[layer.group]
+        xf = x.float()
+        off = 0
+        for b, n in enumerate(step.q_lens):
+            start = step.start_pos[b]
+            pos = torch.arange(start, start + n, device=x.device)
+            rows = table[b].long()
+            if layer.owns_cache:
+                pages[rows[pos // bs], pos % bs] = xf[off:off + n] @ self.wc.T
+            seen = torch.arange(start + n, device=x.device)
+            latents = pages[rows[seen // bs], seen % bs]                     # [ctx, rank]
+            scores = (xf[off:off + n] @ self.wq.T) @ latents.T / math.sqrt(self.rank)
+            scores = scores.masked_fill(seen[None, :] > pos[:, None], float("-inf"))
+            residual[off:off + n] += (torch.softmax(scores, -1) @ latents) @ self.wo.T
+            off += n
+
+
+@dataclass
+class LatentConfig(ModelConfig):
+    hidden_size: int = 0
+    rank: int = 0
+    num_heads: int = 0
+    head_dim: int = 0
+    inter: int = 0
+
+    _KEYS = ("vocab_size", "max_position_embeddings", "hidden_size", "rank", "num_heads", "head_dim", "inter")
+
+    @classmethod
+    def from_dict(cls, d: dict[str, Any]) -> "LatentConfig":
+        return cls(architecture=d["architectures"][0], **{k: d[k] for k in cls._KEYS})
+
+    def to_dict(self) -> dict[str, Any]:
+        return {"architectures": [self.architecture], **{k: getattr(self, k) for k in self._KEYS}}
+
+
+def build_latent(cfg: LatentConfig) -> ModelSpec:
+    h = cfg.hidden_size
+    rot = RotaryPositions(cfg.head_dim, 100.0)
+    latent = kvforge_amd.registry.MIXERS["toy_latent"]
+
+    def block(i, mixer):
+        return PreNormBlock(RMSNorm(f"l.{i}.n1", h, 1e-5), mixer, RMSNorm(f"l.{i}.n2", h, 1e-5),
+                            SwiGLU(f"l.{i}.ff", h, cfg.inter))
+    blocks = [block(0, latent("l.0.mix", h, cfg.rank)),
+              block(1, PagedAttention("l.1.att", h, cfg.num_heads, 1, cfg.head_dim, rot)),
+              block(2, latent("l.2.mix", h, cfg.rank))]
+    return ModelSpec(config=cfg, embedding=TokenEmbedding("embed", cfg.vocab_size, h), blocks=blocks,
+                     final_norm=RMSNorm("norm", h, 1e-5), head=LMHead("head", cfg.vocab_size, h),
+                     positions=[rot])
+
+
+LATENT = {"architectures": ["ToyLatentForCausalLM"], "vocab_size": 61, "max_position_embeddings": 96,
+          "hidden_size": 32, "rank": 12, "num_heads": 2, "head_dim": 16, "inter": 40}
+
+
+def latent_plain(w, ids):
+    wf = {k: v.float() for k, v in w.items()}
+    T = len(ids)
+    h = wf["embed.weight"][torch.tensor(ids)]
+    cos, sin = plain.rope_cos_sin(torch.arange(T), plain.rope_inv_freq(16, 100.0))
+    cfg = {"num_attention_heads": 2, "num_key_value_heads": 1, "head_dim": 16}
+    causal = torch.ones(T, T).tril().bool()
+
+    def latent(x, p):
+        c, q = x @ wf[p + "c.weight"].T, x @ wf[p + "q.weight"].T
+        scores = (q @ c.T / math.sqrt(12)).masked_fill(~causal, float("-inf"))
+        return (torch.softmax(scores, -1) @ c) @ wf[p + "o.weight"].T
+
+    for i in range(3):
+        a = plain.rms_norm(h, wf[f"l.{i}.n1.weight"], 1e-5)
+        h = h + (plain.attention_block(a, wf, "l.1.att.", cfg, cos, sin, None) if i == 1
+                 else latent(a, f"l.{i}.mix."))
+        m = plain.rms_norm(h, wf[f"l.{i}.n2.weight"], 1e-5)
+        h = h + plain.swiglu(m, wf[f"l.{i}.ff.gate_proj.weight"], wf[f"l.{i}.ff.up_proj.weight"],
+                             wf[f"l.{i}.ff.down_proj.weight"])
+    return plain.rms_norm(h, wf["norm.weight"], 1e-5) @ wf["head.weight"].T
+
+
+@pytest.fixture(scope="module")
+def latent_folder(tmp_path_factory):
+    kvforge_amd.register_mixer("toy_latent", ToyLatentMixer)
+    kvforge_amd.register_architecture("ToyLatentForCausalLM", LatentConfig, build_latent)
+    folder = str(tmp_path_factory.mktemp("toy_latent"))
+    kvforge_amd.write_random_model(folder, LATENT, seed=21)
+    return folder
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_mixer_with_pages_of_its_own_make(latent_folder, dtype):
+    w = kvforge_amd.read_safetensors_folder(latent_folder)
+    model = Transformer.from_folder(latent_folder, dtype, DEV)
+    # two groups: the two latent layers share one make of page, attention has another
+    made = {tuple(t.name for t in g.pages): g.layers for g in model.cache_groups}
+    assert made == {("latent",): (0, 2), ("k", "v"): (1,)}
+    bs = 4
+    elem = 4 if dtype == torch.float32 else 2
+    assert bytes_per_block(model.cache_groups, bs, dtype) == 2 * bs * 12 * 4 + 2 * bs * 1 * 16 * elem
+    runner = ModelRunner(model, bs, 20, max_num_seqs=3, max_num_batched_tokens=64, max_model_len=96)
+    assert not runner.use_graphs                         # the toy mixer looks at the step's host fields
+    store = runner.storage.pages
+    assert store[0]["latent"].shape == (20, bs, 12) and store[0]["latent"].dtype == torch.float32
+    assert store[1]["k"].shape == (20, 1, bs, 16) and store[1]["v"].shape == (20, 1, 16, bs)
+    assert store[1]["k"].dtype == dtype and set(store[2]) == {"latent"}
+    g = torch.Generator().manual_seed(3)
+    seqs = {r: torch.randint(0, 61, (n,), generator=g).tolist() for r, n in (("a", 41), ("b", 22), ("c", 30))}
+    want = {r: latent_plain(w, ids) for r, ids in seqs.items()}
+    got = {r: [] for r in seqs}
+    # 20 pages of 4 tokens: a (41) and b (22) together take 17; c (30) needs 8 and gets b's
+    plan = [[("a", 0, 9), ("b", 0, 22)], [("a", 9, 11)], [("a", 11, 40), ("c", 0, 1)],
+            [("a", 40, 41), ("c", 1, 29)], [("c", 29, 30)]]
+    for portions in plan:
+        entries = []
+        for rid, a, b in portions:
+            if not runner.cache.has_request(rid):
+                runner.cache.allocate(rid, 0)
+            runner.cache.append_slots(rid, b, a)
+            entries.append(StepEntry(rid, seqs[rid][a:b], a, "all"))
+        logits = runner.step(entries).cpu()
+        off = 0
+        for rid, a, b in portions:
+            got[rid].append(logits[off:off + b - a])
+            off += b - a
+            if b == len(seqs[rid]):
+                runner.cache.free(rid)
+    t = dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=4e-2)
+    for rid in seqs:
+        torch.testing.assert_close(torch.cat(got[rid]), want[rid], **t)
+    assert runner.cache.num_free_blocks == 20
+
+
+def test_the_latent_model_generates_through_the_engine(latent_folder):
+    w = kvforge_amd.read_safetensors_folder(latent_folder)
+    engine = kvforge_amd.InferenceEngine.from_folder(
+        latent_folder, kvforge_amd.EngineConfig(
+            dtype="float32", cache=kvforge_amd.CacheConfig(block_size=4, num_blocks=48),
+            scheduler=kvforge_amd.SchedulerConfig(max_num_seqs=3, max_num_batched_tokens=8)))
+    prompts = [[5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15], [60, 3], [44, 45, 46, 47, 48]]
+    outs = engine.generate(prompts, kvforge_amd.SamplingParams(max_tokens=9, temperature=0.0))
+    for p, o in zip(prompts, outs):
+        logits = latent_plain(w, p + o.output_token_ids)
+        for i, tok in enumerate(o.output_token_ids):
+            row = logits[len(p) - 1 + i]
+            assert float(row.max() - row[tok]) <= 1e-4
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
