@@ -24,6 +24,16 @@
 //   rotary pairs; rotated q goes to the output (bf16, q heads only), rotated k and plain v go
 //   straight into the pages of the token's sequence (K pages [nb, KV, block, d], V pages
 //   transposed [nb, KV, d, block]).
+// 5 greedy pick for the output head of a decode step (at most 16 bf16 rows, already normalised:
+//   with the norm folded in, each of the head's thousands of workgroups would read the fp32 rows
+//   and their sums of squares again, as many bytes as the matrix itself): no logits are stored;
+//   every workgroup leaves the best (value, column) of its columns per row in a workspace and
+//   takes a ticket, and the workgroup that takes the last one picks every row's best over all
+//   workgroups (the lowest column among equal values), then does what the step's tail would
+//   need kernels of their own for: it hands the tokens out, makes each sequence's token its
+//   next input (token id, position and context length move on by one), keeps the tokens in the
+//   ring row of this step for the host, and writes the tokens' embedding rows into the residual
+//   stream for the next step.
 // K must be a multiple of 8 (16-byte loads); a k-step that passes K loads zeros.
 //
 // A product that is added to a narrow C over a long K (the down projection) has fewer workgroups
@@ -66,6 +76,133 @@ struct Riders {
   const float* c_add;
   float* half_out;
 };
+
+// Operands of the greedy pick (EPI 5).  part_val / part_idx: [16][workgroups] and behind them
+// [16][PICK_LANES] scratch; ticket:
+// PICK_TICKET_INTS ints, zero between launches (atomics on one address are served one after the
+// other, some 65 ns each on this chip, and thousands of workgroups on one counter would queue
+// for longer than the product takes: the workgroups are spread over PICK_LANES counters, a
+// cache line apart, and the last arrival at each takes a ticket of a second counter).  tokens: [M] out.  token_ids / positions / ctx_lens: the step's
+// inputs, advanced in place; ring [ring_rows][ring_stride] and run_counter as decode_advance
+// takes them.  embed [vocab][hidden] bf16 -> residual [M][ld_res] fp32 for the next step.
+struct PickEpi {
+  float* part_val;
+  int* part_idx;
+  int* ticket;
+  int* tokens;
+  int* token_ids;
+  int* positions;
+  int* ctx_lens;
+  int* ring;
+  int* run_counter;
+  const bf16_t* embed;
+  float* residual;
+  int ring_stride, ring_rows, hidden, ld_res;
+};
+
+constexpr int PICK_LANES = 64, PICK_STRIDE = 16;   // counters, and ints between two of them
+constexpr int PICK_TICKET_INTS = (PICK_LANES + 1) * PICK_STRIDE;
+
+// True in the caller (one thread asks) that arrives last of `expected` at `counter`, which it
+// leaves zero.  Every caller has made its results visible before.
+__device__ __forceinline__ bool pick_last_at(int* counter, int expected) {
+  if (atomicAdd(counter, 1) != expected - 1) return false;
+  __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return true;
+}
+
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+  return v > bv || (v == bv && i < bi);
+}
+
+// Results that other workgroups are going to read are stored past this XCD's L2 (an atomic store
+// at device scope is written through); before a ticket is taken they only have to be complete.
+// A device-scope release fence would also write the whole L2's dirty lines back, and thousands
+// of workgroups doing that made the head's product take 275 us instead of 90.
+__device__ __forceinline__ void pick_publish(float* val, int* idx, size_t at, float v, int i) {
+  __hip_atomic_store(val + at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(idx + at, i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void pick_stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+
+// The last arrival at counter `lane`: the best per row over the workgroups lane, lane + 64, ...
+// into the second level of the scratch ([16][PICK_LANES] behind the first).  All threads of the
+// workgroup; plain loads after the caller's acquire fence.
+__device__ __forceinline__ void pick_merge_lane(const PickEpi& pk, int M, int groups, int lane) {
+  const int tid = threadIdx.x, sub = tid % 32;    // 32 threads per row, rows in turn
+  for (int row = tid / 32; row < 16; row += blockDim.x / 32) {   // the same trips in every thread
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    if (row < M) {
+      for (int c = lane + sub * PICK_LANES; c < groups; c += 32 * PICK_LANES) {
+        const float v = pk.part_val[row * groups + c];
+        const int i = pk.part_idx[row * groups + c];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+      }
+    }
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, KVF_WAVE);
+      const int oi = __shfl_xor(bi, o, KVF_WAVE);
+      if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (sub == 0 && row < M)
+      pick_publish(pk.part_val + 16 * groups, pk.part_idx + 16 * groups, row * PICK_LANES + lane, bv, bi);
+  }
+  pick_stores_done();
+}
+
+// The last workgroup of a greedy pick: see EPI 5 at the head of the file.  `lds` holds at least
+// 16 ints.
+__device__ __forceinline__ void pick_finish(const PickEpi& pk, int M, int groups, float* lds) {
+  const int tid = threadIdx.x;
+  const int lanes = groups < PICK_LANES ? groups : PICK_LANES;
+  int* tok = reinterpret_cast<int*>(lds);   // [16]
+  // 16 threads per row over the second level's (at most 64) candidates, rows in turn
+  for (int row = tid / 16; row < 16; row += blockDim.x / 16) {
+    const int sub = tid % 16;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    if (row < M) {
+      for (int c = sub; c < lanes; c += 16) {
+        const float v = pk.part_val[16 * groups + row * PICK_LANES + c];
+        const int i = pk.part_idx[16 * groups + row * PICK_LANES + c];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+      }
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, KVF_WAVE);
+      const int oi = __shfl_xor(bi, o, KVF_WAVE);
+      if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (sub == 0 && row < M) tok[row] = bi == 0x7fffffff ? 0 : bi;
+  }
+  const int step = *pk.run_counter;   // read by every thread before it moves
+  __syncthreads();
+  if (tid < M) {
+    const int t = tok[tid];
+    pk.tokens[tid] = t;
+    if (step >= 0 && step < pk.ring_rows) pk.ring[step * pk.ring_stride + tid] = t;
+    if (pk.ctx_lens[tid] > 0) {     // padding sequences stay empty
+      pk.token_ids[tid] = t;
+      pk.positions[tid] += 1;
+      pk.ctx_lens[tid] += 1;
+    }
+  }
+  if (tid == 0) *pk.run_counter = step + 1;
+  __syncthreads();
+  // the tokens' embedding rows, widened, are the next step's residual stream
+  const int per_row = pk.hidden / 8;
+  for (int idx = tid; idx < M * per_row; idx += blockDim.x) {
+    const int r = idx / per_row, k = (idx - r * per_row) * 8;
+    float v[8];
+    load8(pk.embed + static_cast<size_t>(tok[r]) * pk.hidden + k, v);
+    float* dst = pk.residual + static_cast<size_t>(r) * pk.ld_res + k;
+    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(dst + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+}
 
 __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
   uint4 r = make_uint4(0u, 0u, 0u, 0u);
@@ -241,7 +378,7 @@ constexpr int depth(int mt, int nt, int at) {
 template <int MT, int NT, int AT, int EPI, bool ADD>
 __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_kernel(
     const void* __restrict__ Av, const bf16_t* __restrict__ W, void* __restrict__ Cv, int M, int N,
-    int K, int lda, int ldc, int m_base, float eps, int w_tiled, Riders rd, RopeEpi rp) {
+    int K, int lda, int ldc, int m_base, float eps, int w_tiled, Riders rd, RopeEpi rp, PickEpi pk) {
   constexpr int RW = 16;  // rows of W per group
   extern __shared__ float red[];  // [nw][MT][64 lanes][4], then [nw][MT][16] sums of squares
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
@@ -359,6 +496,8 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
     }
   }
   // lane holds C[row r16][cols n0 + 16*j + 4*kg .. +3] of each tile
+  float pick_v = -INFINITY;   // EPI 5: the best of this thread's columns of its row so far
+  int pick_i = 0x7fffffff;
   float* red_ss = red + nw * MT * KVF_WAVE * 4;
   if (AT) {
 #pragma unroll
@@ -389,6 +528,12 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
         for (int w = 0; w < nw; ++w) tot += red_ss[(w * MT + t) * 16 + l % 16];
         s *= rsqrtf(tot / static_cast<float>(K) + eps);
       }
+      if (EPI == 5) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (n + r < N && better(s[r], n + r, pick_v, pick_i)) { pick_v = s[r]; pick_i = n + r; }
+        continue;
+      }
       EpiOperands fresh;
       fresh.have = false;
       if (EPI == 2 && second)
@@ -396,6 +541,41 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       else
         store_tile<EPI>(s, m, n, N, ldc, Cv, c_add, rp, PRE ? pre[j] : fresh);
     }
+  }
+  if (EPI == 5) {
+    // one row tile: the first 64 threads hold row r16's best over their four columns of every
+    // group of this workgroup
+    if (wave == 0) {
+#pragma unroll
+      for (int o = 16; o <= 32; o <<= 1) {
+        const float ov = __shfl_xor(pick_v, o, KVF_WAVE);
+        const int oi = __shfl_xor(pick_i, o, KVF_WAVE);
+        if (better(ov, oi, pick_v, pick_i)) { pick_v = ov; pick_i = oi; }
+      }
+      const int m = m_base + r16;
+      if (kg == 0 && m < M)
+        pick_publish(pk.part_val, pk.part_idx, static_cast<size_t>(m) * gridDim.x + blockIdx.x, pick_v, pick_i);
+      pick_stores_done();
+    }
+    // Two levels of tickets: the workgroups are spread over PICK_LANES counters; the last
+    // arrival at a counter merges that counter's workgroups and takes a ticket of the top
+    // counter; the last arrival there finishes.
+    const int groups = static_cast<int>(gridDim.x), lane_id = static_cast<int>(blockIdx.x) % PICK_LANES;
+    int* flag = reinterpret_cast<int*>(red);
+    __syncthreads();     // (and nobody reads `red` any more)
+    if (threadIdx.x == 0)
+      flag[0] = pick_last_at(pk.ticket + lane_id * PICK_STRIDE, (groups - lane_id + PICK_LANES - 1) / PICK_LANES);
+    __syncthreads();
+    if (flag[0] == 0) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // what the others published, not this XCD's stale copy
+    pick_merge_lane(pk, M, groups, lane_id);
+    __syncthreads();
+    if (threadIdx.x == 0)
+      flag[1] = pick_last_at(pk.ticket + PICK_LANES * PICK_STRIDE, groups < PICK_LANES ? groups : PICK_LANES);
+    __syncthreads();
+    if (flag[1] == 0) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    pick_finish(pk, M, groups, red + 64);
   }
 }
 
@@ -415,23 +595,25 @@ int pick_waves(int K) {
 
 template <int MT, int NT, int AT, int EPI>
 int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
-               int m_base, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
+               int m_base, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s,
+               const PickEpi& pk = PickEpi{}) {
   const int groups = (N + 16 * NT - 1) / (16 * NT);
   int nw = pick_waves(K);
   if (nw > max_waves(MT, NT, AT)) nw = max_waves(MT, NT, AT);
   const dim3 grid(groups, EPI == 2 && rd.half_out ? 2 : 1), block(nw * KVF_WAVE);
-  const size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
+  size_t lds = static_cast<size_t>(nw) * MT * (KVF_WAVE * 4 + 16) * sizeof(float);
+  if (EPI == 5 && lds < (64 + 2 * 16 * 16 + 16) * sizeof(float)) lds = (64 + 2 * 16 * 16 + 16) * sizeof(float);
   if (rd.a_add) {
     // the sum that rides in the left operand's loads: only the fused q/k/v projection of one
     // tile of rows is built with it
     if constexpr (MT == 1 && AT == 1 && EPI == 4)
       hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, true>), grid, block, lds, s, A, W, C, M, N, K,
-                         lda, ldc, m_base, eps, w_tiled, rd, rp);
+                         lda, ldc, m_base, eps, w_tiled, rd, rp, pk);
     else
       return static_cast<int>(hipErrorInvalidValue);
   } else {
     hipLaunchKernelGGL((gemm_skinny_kernel<MT, NT, AT, EPI, false>), grid, block, lds, s, A, W, C, M, N, K,
-                       lda, ldc, m_base, eps, w_tiled, rd, rp);
+                       lda, ldc, m_base, eps, w_tiled, rd, rp, pk);
   }
   return kvf_last_error();
 }
@@ -539,4 +721,37 @@ KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, 
   if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);
   if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);
   return static_cast<int>(hipErrorInvalidValue);
+}
+
+
+// How many workgroups the greedy pick of M rows over N columns launches: the caller sizes
+// part_val / part_idx as 16 * that many.
+KVF_EXPORT int kvf_gemm_bf16_pick_ticket_ints() { return PICK_TICKET_INTS; }
+KVF_EXPORT int kvf_gemm_bf16_pick_groups(int M, int N) {
+  const int tiles = (N + 15) / 16;
+  const int nt = (M > 4 && tiles >= 512) ? 2 : 1;
+  return (N + 16 * nt - 1) / (16 * nt);
+}
+
+// Output head of a decode step with the greedy pick and the step's tail folded in (EPI 5 at the
+// head of the file).  A: the normalised rows [M <= 16, lda] bf16.  W: [N, K] bf16, row-major or
+// tiled.  residual: [M, ld_res] fp32, receives the picked tokens' rows of `embed` [>= N, hidden].
+// See PickEpi for the rest.
+KVF_EXPORT int kvf_gemm_bf16_pick(const void* A, const void* W, int w_tiled, int M, int N, int K,
+                                  int lda, float* part_val, int* part_idx, int* ticket, int* tokens,
+                                  int* token_ids, int* positions, int* ctx_lens, int* ring,
+                                  int* run_counter, int ring_stride, int ring_rows, const void* embed,
+                                  float* residual, int hidden, int ld_res, hipStream_t s) {
+  if (M <= 0) return 0;
+  if (M > 16 || N <= 0 || K <= 0 || K % 8 != 0 || lda % 8 != 0 || hidden % 8 != 0 || ld_res % 4 != 0 ||
+      ring_stride < M || ring_rows <= 0 || !part_val || !part_idx || !ticket)
+    return static_cast<int>(hipErrorInvalidValue);
+  const Riders rd{nullptr, nullptr, nullptr};
+  const RopeEpi none{};
+  const PickEpi pk{part_val, part_idx, ticket, tokens, token_ids, positions, ctx_lens, ring, run_counter,
+                   static_cast<const bf16_t*>(embed), residual, ring_stride, ring_rows, hidden, ld_res};
+  const bf16_t* w = static_cast<const bf16_t*>(W);
+  if (M > 4 && (N + 15) / 16 >= 512)   // two groups of 16 columns per workgroup, as pick_groups counts
+    return launch_one<1, 2, 0, 5>(A, w, nullptr, M, N, K, lda, 0, 0, 0.f, w_tiled, rd, none, s, pk);
+  return launch_one<1, 1, 0, 5>(A, w, nullptr, M, N, K, lda, 0, 0, 0.f, w_tiled, rd, none, s, pk);
 }

@@ -31,6 +31,20 @@ class DecodeShape:
 
 
 @dataclass
+class DecodeTail:
+    """What the head's greedy pick needs besides the step to do the tail of a decode step by
+    itself (``Transformer.forward(step, tail=...)``): where the picked tokens go, the ring and
+    the counter of the run's steps, the embedding table for the next step's residual stream,
+    and the pick's scratch."""
+
+    tokens: torch.Tensor
+    ring: torch.Tensor
+    run_counter: torch.Tensor
+    embed_table: torch.Tensor
+    work: tuple
+
+
+@dataclass
 class StepEntry:
     """``want``: places among ``token_ids`` whose logits are returned, or ``"last"`` / ``"all"``
     / ``"none"`` (the reference's ``LogitsMode``)."""

@@ -16,8 +16,8 @@ import torch
 
 from kvforge_amd.cache.manager import CacheManager
 from kvforge_amd.cache.storage import PagedStorage, StateStorage, bytes_per_block
-from kvforge_amd.engine.batch import (DecodeShape, MetaBuffers, Step, StepEntry, Workspace,
-                                      extend_tables, fill_step)
+from kvforge_amd.engine.batch import (DecodeShape, DecodeTail, MetaBuffers, Step, StepEntry,
+                                      Workspace, extend_tables, fill_step)
 from kvforge_amd.kernels import ops
 from kvforge_amd.sampling.rng import uniform
 from kvforge_amd.kernels import library
@@ -79,6 +79,14 @@ class ModelRunner:
         self._sample_rows: list[tuple] = []
         self._sample_bucket = 0
         self._sample_drawn: list[int] = []
+        # Steps whose rows are all picked greedily end in the head's own kernel (no logits, no
+        # sampling, advance or embedding kernels) where the model allows it.
+        self.num_greedy_tails = 0
+        self._tail: DecodeTail | None = None
+        if self.use_graphs and model.can_pick(1):
+            self._tail = DecodeTail(self._sample_i[cap:2 * cap], self._run_ring, self._run_counter,
+                                    model.spec.embedding.table,
+                                    ops.pick_workspace(16, model.config.vocab_size, self.device))
 
     @staticmethod
     def bytes_per_block(model: Transformer, block_size: int) -> int:
@@ -242,24 +250,29 @@ class ModelRunner:
         if dirty:
             self._sample_f.copy_(self._sample_f_host, non_blocking=True)
         self._run_counter.zero_()
-        key = (bucket, launch_key)
+        greedy = self._tail is not None and not self._sample_drawn and self.model.can_pick(bucket)
+        key = (bucket, launch_key, greedy)
         graph = self.graphs.get(key)
         replays = k
+        if greedy:
+            # the run's first residual stream; every later one is left there by the step before
+            self.model.embed(step)
+            self.num_greedy_tails += k
         if graph is None:
-            self._forward_and_sample(step, bucket)          # the first step, and a warm-up
-            graph = self.graphs[key] = self._capture(step, bucket)
+            self._forward_and_sample(step, bucket, greedy)  # the first step, and a warm-up
+            graph = self.graphs[key] = self._capture(step, bucket, greedy)
             replays -= 1
         for _ in range(replays):
             graph.graph.replay()
-        return self._queue_read(ids, [e.start_pos for e in entries], k, 0, bucket, replays)
+        return self._queue_read(ids, [e.start_pos for e in entries], k, 0, bucket, replays, greedy)
 
-    def _queue_read(self, ids, begins, k: int, base: int, bucket: int, replays: int
-                    ) -> "_QueuedRun":
+    def _queue_read(self, ids, begins, k: int, base: int, bucket: int, replays: int,
+                    greedy: bool = False) -> "_QueuedRun":
         """Queue the copy of ring rows ``base..base+k-1`` to the host behind the run's launches."""
         self._ring_host[base:base + k].copy_(self._run_ring[base:base + k], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        return _QueuedRun(ids, begins, k, base, bucket, replays, event)
+        return _QueuedRun(ids, begins, k, base, bucket, replays, event, greedy)
 
     def _continue_run(self, run: "_QueuedRun", entries, seed, streams, counters
                       ) -> "_QueuedRun | None":
@@ -270,7 +283,7 @@ class ModelRunner:
         if any(s + k > self.max_model_len for s in starts):
             return None
         shape = DecodeShape(len(starts), max(starts) + 1, sum(s + 1 for s in starts))
-        graph = self.graphs.get((run.bucket, self.model.launch_key(shape)))
+        graph = self.graphs.get((run.bucket, self.model.launch_key(shape), run.greedy))
         if graph is None:
             return None
         base = k if run.base == 0 else 0
@@ -293,9 +306,15 @@ class ModelRunner:
             self._run_counter.zero_()
         for _ in range(k):
             graph.graph.replay()
-        return self._queue_read(run.ids, starts, k, base, run.bucket, k)
+        self.num_greedy_tails += k if run.greedy else 0
+        return self._queue_read(run.ids, starts, k, base, run.bucket, k, run.greedy)
 
-    def _forward_and_sample(self, step: Step, rows: int) -> torch.Tensor:
+    def _forward_and_sample(self, step: Step, rows: int, greedy: bool = False) -> torch.Tensor | None:
+        """One decode step of a padded batch with everything up to its next inputs.  ``greedy``:
+        all rows take the largest logit and the residual stream is in place already: the head's
+        kernel does the whole tail."""
+        if greedy:
+            return self.model.forward(step, tail=self._tail, embedded=True)
         cap = self.meta.max_seqs
         logits = self.model.forward(step)
         sampled = self._sample_i[cap:cap + rows]
@@ -306,13 +325,13 @@ class ModelRunner:
                            self._run_counter)
         return logits
 
-    def _capture(self, step: Step, rows: int) -> "_DecodeGraph":
+    def _capture(self, step: Step, rows: int, greedy: bool = False) -> "_DecodeGraph":
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         self.ws.frozen = True
         try:
             with torch.cuda.graph(graph):
-                logits = self._forward_and_sample(step, rows)
+                logits = self._forward_and_sample(step, rows, greedy)
         finally:
             self.ws.frozen = False
         # the graph keeps the workspace it was recorded with alive, whatever grows later
@@ -328,9 +347,9 @@ class _QueuedRun:
     begins them at, which ring rows hold their tokens, and the event behind the copy of those
     rows."""
 
-    def __init__(self, ids, begins, k, base, bucket, replays, event) -> None:
+    def __init__(self, ids, begins, k, base, bucket, replays, event, greedy=False) -> None:
         self.ids, self.begins, self.k, self.base = ids, begins, k, base
-        self.bucket, self.replays, self.event = bucket, replays, event
+        self.bucket, self.replays, self.event, self.greedy = bucket, replays, event, greedy
 
 
 class _DecodeGraph:

@@ -519,6 +519,70 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
           _stream()), "gemm_qkv_rope")
 
 
+def pick_workspace(rows: int, n: int, device) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Scratch of ``gemm_pick`` for ``rows`` rows over ``n`` columns: the workgroups' best values
+    and columns, and the ticket (one int, zero between launches)."""
+    pick_groups = _fn("gemm_bf16", "kvf_gemm_bf16_pick_groups", [c_int, c_int])
+    # few rows take fewer columns per workgroup, hence more workgroups: room for any count up to rows
+    groups = max(int(pick_groups(m, int(n))) for m in range(1, int(rows) + 1))
+    tickets = int(_fn("gemm_bf16", "kvf_gemm_bf16_pick_ticket_ints", [])())
+    return (torch.empty(16 * groups + 16 * 64, dtype=F32, device=device),
+            torch.empty(16 * groups + 16 * 64, dtype=I32, device=device),
+            torch.zeros(tickets, dtype=I32, device=device))
+
+
+def gemm_pick(a: torch.Tensor, w, residual: torch.Tensor, tokens: torch.Tensor,
+              token_ids: torch.Tensor, positions: torch.Tensor, ctx_lens: torch.Tensor,
+              ring: torch.Tensor, run_counter: torch.Tensor, embed: torch.Tensor, work: tuple) -> None:
+    """The output head of a decode step with everything after it folded in: ``a`` (the
+    normalised rows, bf16, at most 16, one per sequence) is multiplied by ``w``, the largest
+    logit of every row is picked without the logits being stored (lowest column among equal
+    ones), and the picked token becomes its sequence's next input exactly as ``decode_advance``
+    does it; the tokens' rows of ``embed`` are then written into ``residual`` (fp32, a row per
+    sequence) as the next step's residual stream.  ``work``: from ``pick_workspace``; launches
+    that share it must not overlap."""
+    m, k = a.shape
+    _check(a, "a", BF16, (m, k), contiguous=False)
+    if a.stride(1) != 1 or m > FUSED_NORM_MAX_M or m == 0:
+        raise KernelError(f"gemm_pick takes 1 to {FUSED_NORM_MAX_M} dense bf16 rows")
+    _check(plain_of(w), "w", BF16, (None, k))
+    n = w.shape[0]
+    if not bf16_kernel_takes(a, w):
+        raise KernelError("gemm_pick: operands do not fit the MFMA kernel")
+    _check(residual, "residual", F32, (m, k), contiguous=False)
+    if residual.stride(1) != 1 or (m > 1 and residual.stride(0) % 4):
+        raise KernelError("gemm_pick: rows of the residual stream must be dense and start on 16 bytes")
+    for t, name in ((tokens, "tokens"), (token_ids, "token_ids"), (positions, "positions"),
+                    (ctx_lens, "ctx_lens")):
+        _check(t, name, I32, (None,))
+        if t.shape[0] < m:
+            raise KernelError(f"gemm_pick: {name} is shorter than the batch")
+    _check(ring, "ring", I32, (None, None))
+    _check(run_counter, "run_counter", I32, (1,))
+    if ring.shape[1] < m:
+        raise KernelError("gemm_pick: rows of the ring are shorter than the batch")
+    _check(embed, "embed", BF16, (None, k))
+    if embed.shape[0] < n or k % 8:
+        raise KernelError("gemm_pick: the embedding table must hold a row of K elements (a multiple "
+                          "of 8) for every column of w")
+    part_val, part_idx, ticket = work
+    groups = int(_fn("gemm_bf16", "kvf_gemm_bf16_pick_groups", [c_int, c_int])(m, n))
+    _check(part_val, "work[0]", F32, (None,))
+    _check(part_idx, "work[1]", I32, (None,))
+    _check(ticket, "work[2]", I32, (int(_fn("gemm_bf16", "kvf_gemm_bf16_pick_ticket_ints", [])()),))
+    if part_val.shape[0] < 16 * groups + 16 * 64 or part_idx.shape[0] < 16 * groups + 16 * 64:
+        raise KernelError("gemm_pick: workspace too small for these rows and columns")
+    f = _fn("gemm_bf16", "kvf_gemm_bf16_pick",
+            [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 9
+            + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p])
+    wp, tiled = _w_args(w)
+    _ok(f(a.data_ptr(), wp, tiled, m, n, k, a.stride(0) if m > 1 else k, part_val.data_ptr(),
+          part_idx.data_ptr(), ticket.data_ptr(), tokens.data_ptr(), token_ids.data_ptr(),
+          positions.data_ptr(), ctx_lens.data_ptr(), ring.data_ptr(), run_counter.data_ptr(),
+          ring.shape[1], ring.shape[0], embed.data_ptr(), residual.data_ptr(), k,
+          residual.stride(0) if m > 1 else k, _stream()), "gemm_pick")
+
+
 def set_gemm_waves(waves: int, rows: int = 0) -> None:
     """Measurement aid: force the waves per workgroup and the rows of W per workgroup of the
     MFMA kernel (0 = by shape)."""

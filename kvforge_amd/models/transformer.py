@@ -9,7 +9,7 @@ import torch
 from kvforge_amd import registry
 from kvforge_amd.cache.manager import CacheGroup
 from kvforge_amd.kernels import library
-from kvforge_amd.parts.base import Block, CacheSpec, LayerState, ModelSpec, StateSpec
+from kvforge_amd.parts.base import Block, CacheSpec, LayerState, ModelSpec, Positions, StateSpec
 from kvforge_amd.weights.loader import load_model_weights
 
 
@@ -67,13 +67,14 @@ class Transformer:
         cfg = registry.config_from_dict(config) if isinstance(config, dict) else config
         model = cls(registry.build_spec(cfg), dtype, device)
         load_random_weights(model.spec, seed, dtype, device)
-        for p in model.spec.all_parts():
-            p.seal()
-        model._loaded = True
+        model._seal()
         return model
 
     def load_folder(self, folder: str) -> None:
         load_model_weights(self.spec, folder, self.dtype, self.device)
+        self._seal()
+
+    def _seal(self) -> None:
         for p in self.spec.all_parts():
             p.seal()
         self._loaded = True
@@ -131,25 +132,58 @@ class Transformer:
         return sum(seen.values())
 
     # ------------------------------------------------------------------ forward
-    def forward(self, step) -> torch.Tensor:
-        """Runs the step's tokens from the cache; returns fp32 logits ``[n_logits, vocab]`` (a
-        view of workspace memory, valid until the next forward)."""
+    def can_pick(self, rows: int) -> bool:
+        """Whether a decode step of ``rows`` sequences can end in the head's greedy pick
+        (``forward(step, tail=...)``): the head streams a bf16 matrix, the embedding is a plain
+        bf16 table and no position encoding touches the embedding output."""
         spec = self.spec
-        cfg = self.config
-        hidden = spec.embedding.hidden
-        residual = step.ws.buf("residual", (step.n_tokens, hidden), torch.float32)
+        table = getattr(spec.embedding, "table", None)
+        plain_embedding = (type(spec.embedding).__name__ == "TokenEmbedding" and table is not None
+                           and table.dtype == torch.bfloat16)
+        untouched = all(type(p).on_embedding is Positions.on_embedding for p in spec.positions)
+        return (self.dtype == torch.bfloat16 and plain_embedding and untouched
+                and hasattr(spec.head, "can_pick") and spec.head.can_pick(rows))
+
+    def embed(self, step) -> torch.Tensor:
+        """The step's residual stream, filled from the embedding."""
+        spec = self.spec
+        residual = step.ws.buf("residual", (step.n_tokens, spec.embedding.hidden), torch.float32)
         spec.embedding.forward(step.token_ids, residual)
         for p in spec.positions:
             p.on_embedding(residual, step)
+        return residual
+
+    def forward(self, step, tail=None, embedded: bool = False) -> torch.Tensor | None:
+        """Runs the step's tokens from the cache; returns fp32 logits ``[n_logits, vocab]`` (a
+        view of workspace memory, valid until the next forward).
+
+        ``tail`` (a ``DecodeTail``, for a step of single tokens that all want their logits and
+        are picked greedily, where ``can_pick`` allows it): no logits are made; the head's
+        kernel picks the tokens, makes them the sequences' next inputs and leaves their
+        embeddings in the residual stream, so that the next such step runs with ``embedded``
+        (the stream is there already) and returns ``None`` again."""
+        spec = self.spec
+        cfg = self.config
+        hidden = spec.embedding.hidden
+        if embedded:
+            residual = step.ws.buf("residual", (step.n_tokens, hidden), torch.float32)
+        else:
+            residual = self.embed(step)
         for call, ls in zip(self.order, self.layer_states):
             spec.blocks[call.layer].forward(residual, step, ls)
         r = step.n_logits
+        if tail is not None and (r != step.n_tokens or not self.can_pick(r)):
+            raise ValueError("the greedy tail is for steps of single tokens that all want their "
+                             "logits, on a model that can_pick")
         if r == 0:
             step.owed = None
             return torch.empty((0, cfg.vocab_size), dtype=torch.float32, device=residual.device)
         x = step.ws.buf("final_normed", (r, hidden), step.act_dtype)
         # only the wanted rows matter now: what is still owed to the stream is added to them alone
         spec.final_norm.forward(residual, x, step.logits_rows, add=step.take_owed(residual))
+        if tail is not None:
+            spec.head.pick(x, residual, step, tail)
+            return None
         logits = step.ws.buf("logits", (r, cfg.vocab_size), torch.float32)
         spec.head.forward(x, logits)
         return logits

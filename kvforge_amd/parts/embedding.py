@@ -67,3 +67,14 @@ class LMHead(Part):
 
     def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
         ops.gemm(x, self.weight, logits)
+
+    def can_pick(self, rows: int) -> bool:
+        """Whether ``pick`` takes so many rows with this weight."""
+        return (isinstance(self.weight, ops.StreamedWeight) and 0 < rows <= ops.FUSED_NORM_MAX_M
+                and self.hidden % 8 == 0)
+
+    def pick(self, x: torch.Tensor, residual: torch.Tensor, step, tail) -> None:
+        """The tail of a greedy decode step in one kernel (``ops.gemm_pick``): ``x`` holds the
+        normalised row of every sequence, all of them wanted."""
+        ops.gemm_pick(x, self.weight, residual, tail.tokens, step.token_ids, step.positions,
+                      step.ctx_lens, tail.ring, tail.run_counter, tail.embed_table, tail.work)

@@ -716,7 +716,7 @@ def test_graph_replay_of_library_products_at_the_served_width(tmp_path):
 
     eager, _ = run(False)
     graphed, engine = run(True)
-    assert any(b == 64 for b, _ in engine.runner.graphs) and engine.runner.num_graph_replays >= 16
+    assert any(b == 64 for b, *_ in engine.runner.graphs) and engine.runner.num_graph_replays >= 16
     assert graphed == eager
     again, _ = run(True)
     assert again == graphed
@@ -744,7 +744,7 @@ def test_one_long_context_among_short_ones(tmp_path):
         engine = InferenceEngine.from_folder(folder, config)
         outs = [o.output_token_ids for o in engine.generate(prompts, params)]
         if use_graphs:
-            assert any(skew > 1 for _, keys in engine.runner.graphs for _, skew in keys)
+            assert any(skew > 1 for _, keys, _ in engine.runner.graphs for _, skew in keys)
         for i in (0, 1, 7):
             oracle.check_choices(prompts[i], outs[i], 3e-2)
         assert engine.cache.num_free_blocks == engine.cache.num_blocks
@@ -754,8 +754,9 @@ def test_wide_layers_through_graphs_and_queued_runs(tmp_path):
     """A model whose layers are wide enough for the kernels a real model is served with (the down
     projection in two halves of K, one of them owed from layer to layer; two groups of columns
     per wave in gate/up; head size 64 on the matrix cores): six requests in bf16 through captured
-    graphs, runs of steps on the device and runs queued ahead give the tokens of single eager
-    steps, and every token is the plain model's choice within bf16 rounding."""
+    graphs, runs of steps on the device and runs queued ahead give the tokens of single captured
+    steps, and every token, theirs and that of eager steps, is the plain model's choice within
+    bf16 rounding."""
     from tests.replay_util import WIDE, sharpen
     folder = str(tmp_path / "wide")
     kvforge_amd.write_random_model(folder, dict(WIDE), seed=4)
@@ -770,11 +771,19 @@ def test_wide_layers_through_graphs_and_queued_runs(tmp_path):
         return [o.output_token_ids for o in engine.generate(prompts, params)], engine
 
     eager, _ = run(use_graphs=False, decode_run_steps=1)
+    single, _ = run(use_graphs=True, decode_run_steps=1)
     served, engine = run(use_graphs=True, decode_run_steps=8, decode_run_ahead=True)
     assert engine.runner.num_graph_replays > 0 and engine.runner.num_runs_queued_ahead >= 1
-    assert served == eager
-    for p, out in zip(prompts, served):
-        oracle.check_choices(p, out, 3e-2)
+    # captured steps end in the head's greedy pick (no logits, the norm inside the product):
+    # the same kernels whether the device takes one step or runs of them
+    assert engine.runner.num_greedy_tails > 0
+    assert served == single
+    # eager steps make logits and pick from them; the two round differently, so where the plain
+    # model's two best logits lie within bf16 rounding they may part ways: each is held to the
+    # plain model on its own history
+    for p, a, b in zip(prompts, served, eager):
+        oracle.check_choices(p, a, 3e-2)
+        oracle.check_choices(p, b, 3e-2)
 
 
 @pytest.mark.parametrize("count,bucket", [(24, 32), (40, 64)])
@@ -794,7 +803,7 @@ def test_graph_replay_with_many_requests(model_a, count, bucket):
 
     eager, _ = run(False)
     graphed, engine = run(True)
-    assert any(b == bucket for b, _ in engine.runner.graphs) and engine.runner.num_graph_replays >= 8
+    assert any(b == bucket for b, *_ in engine.runner.graphs) and engine.runner.num_graph_replays >= 8
     assert graphed == eager
     for p, out in zip(prompts, graphed):
         oracle.check_choices(p, out, 3e-2)

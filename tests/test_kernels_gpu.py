@@ -198,6 +198,68 @@ def test_gemm_of_many_rows_through_the_library_entry_point(m, n, k):
     torch.testing.assert_close(acc.double().cpu(), res.double() + owed.double() + want, atol=1e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("n,k", [(1000, 256), (128256, 128), (8200, 2048), (37, 64)])
+@pytest.mark.parametrize("tiled", [True, False])
+def test_gemm_pick_is_head_argmax_advance_and_embedding(m, n, k, tiled):
+    """The greedy tail of a decode step in one kernel against its parts done plainly: the
+    normalised rows times the head's matrix, the largest logit's column per row, the sequences'
+    next inputs moved on (padding sequences left alone), the ring row of the step, the step
+    counter, and the tokens' embedding rows as the next residual stream.  Twice in a row over
+    the same scratch."""
+    g = torch.Generator().manual_seed(m * 7 + k)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16)
+    embed = torch.randn(n, k, generator=g).to(torch.bfloat16).to(DEV)
+    sw = ops().StreamedWeight(w.to(DEV)) if tiled else w.to(DEV)
+    work = ops().pick_workspace(16, n, DEV)
+    ring = torch.full((4, 20), -1, dtype=torch.int32, device=DEV)
+    counter = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ctx = torch.tensor([5 + i if i % 4 != 3 else 0 for i in range(m)], dtype=torch.int32)  # some padding
+    for call in range(2):
+        x = torch.randn(m, k + 8, generator=g).to(torch.bfloat16)[:, :k]      # a row stride wider than K
+        logits = x.double() @ w.double().T
+        residual = torch.full((m, k), 3.0, device=DEV)
+        tokens = torch.full((m,), -5, dtype=torch.int32, device=DEV)
+        token_ids = torch.full((m,), 7, dtype=torch.int32, device=DEV)
+        positions = torch.arange(10, 10 + m, dtype=torch.int32, device=DEV)
+        ctx_dev = ctx.clone().to(DEV)
+        wide = torch.zeros(m, k + 8, dtype=torch.bfloat16, device=DEV)
+        wide[:, :k] = x.to(DEV)
+        ops().gemm_pick(wide[:, :k], sw, residual, tokens, token_ids, positions, ctx_dev, ring, counter,
+                        embed, work)
+        got = tokens.cpu()
+        top2 = logits.topk(2, dim=-1).values
+        for r in range(m):
+            if float(top2[r, 0] - top2[r, 1]) > 1e-4:          # fp32 sums of bf16 products: near exact
+                assert int(got[r]) == int(logits[r].argmax()), (call, r)
+            assert float(logits[r].max() - logits[r, int(got[r])]) <= 1e-4
+        live = ctx > 0
+        assert torch.equal(token_ids.cpu()[live], got[live]) and (token_ids.cpu()[~live] == 7).all()
+        assert torch.equal(positions.cpu(), torch.arange(10, 10 + m, dtype=torch.int32) + live.int())
+        assert torch.equal(ctx_dev.cpu(), ctx + live.int())
+        assert int(counter) == call + 1 and torch.equal(ring[call, :m].cpu(), got)
+        assert (ring[call + 1:] == -1).all() and int(work[2].abs().sum()) == 0
+        assert torch.equal(residual.cpu(), embed.float().cpu()[got.long()])
+
+
+def test_gemm_pick_takes_the_lowest_of_equal_columns():
+    """Rows of zeros give equal logits everywhere: column 0 wins in every row, through every
+    workgroup's partial result and the last one's merge."""
+    n, k, m = 50000, 64, 8
+    w = torch.randn(n, k, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(DEV)
+    sw = ops().StreamedWeight(w)
+    a = torch.zeros(m, k, dtype=torch.bfloat16, device=DEV)
+    a[3, 5] = 1.0                                    # one row with a real best column
+    tokens = torch.full((m,), -1, dtype=torch.int32, device=DEV)
+    i32 = lambda v: torch.full((m,), v, dtype=torch.int32, device=DEV)
+    ops().gemm_pick(a, sw, torch.zeros(m, k, device=DEV), tokens, i32(0), i32(0), i32(1),
+                    torch.zeros(2, m, dtype=torch.int32, device=DEV),
+                    torch.zeros(1, dtype=torch.int32, device=DEV), w, ops().pick_workspace(16, n, DEV))
+    want = [0] * m
+    want[3] = int(w[:, 5].float().argmax())
+    assert tokens.tolist() == want
+
+
 @pytest.mark.parametrize("m", [1, 5, 16])
 @pytest.mark.parametrize("n,k", [(352, 96), (40, 2048), (100, 40), (2048, 136), (16, 32)])
 def test_gemm_over_tiled_weights_gives_the_same_bits(m, n, k):
