@@ -394,7 +394,7 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
 }
 
 // One workgroup per (sequence slot, head): the cuts' partial results into the output row, in
-// cut order.  A sequence without context (padding of a captured batch) writes nothing.
+// cut order.  A sequence without context (padding of a captured batch) gets a row of zeros.
 template <typename T>
 __global__ __launch_bounds__(KVF_WAVE) void attn_decode_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
@@ -402,8 +402,13 @@ __global__ __launch_bounds__(KVF_WAVE) void attn_decode_merge_kernel(
     T* __restrict__ out, DecodeArgs a) {
   const int head = blockIdx.x, slot = blockIdx.y;
   const int seq = seq_ids ? seq_ids[slot] : slot;
-  if (seq < 0 || seq >= a.n_seqs || ctx_lens[seq] <= 0) return;
+  if (seq < 0 || seq >= a.n_seqs) return;
   const int token = cu_q ? cu_q[seq] : seq;
+  if (ctx_lens[seq] <= 0) {
+    for (int e = threadIdx.x; e < a.d; e += KVF_WAVE)
+      Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * a.d + e, 0.f);
+    return;
+  }
   const size_t p0 = (static_cast<size_t>(slot) * a.H + head) * a.splits;
   float m = -INFINITY;
   for (int c = 0; c < a.splits; ++c) m = fmaxf(m, part_ml[2 * (p0 + c)]);

@@ -629,14 +629,21 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
 
 // Merges the splits of every (sequence, head) in split order.  One query token per sequence, one
 // wave per (sequence, head), at most 64 splits; the partial maxima are in log2 units.  Lane s
-// weighs split s; the loads of the partial accumulators do not depend on one another.
+// weighs split s; the loads of the partial accumulators do not depend on one another.  A
+// sequence without context (the padding of a captured batch) has no partial results: its row
+// is cleared and the workspace is not read.
 __global__ __launch_bounds__(64) void attn_split_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int* __restrict__ seq_ids, const int* __restrict__ cu_q, bf16_t* __restrict__ out, int H, int D,
-    int splits, int o_stride, int n_seqs) {
+    const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
+    bf16_t* __restrict__ out, int H, int D, int splits, int o_stride, int n_seqs) {
   const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
   if (seq < 0 || seq >= n_seqs) return;
   const int head = blockIdx.y, lane = threadIdx.x;
+  if (ctx_lens[seq] <= 0) {
+    const int token = cu_q ? cu_q[seq] : seq;
+    for (int e = lane; e < D; e += KVF_WAVE) out[static_cast<size_t>(token) * o_stride + head * D + e].bits = 0;
+    return;
+  }
   const size_t slot0 = (static_cast<size_t>(blockIdx.x) * H + head) * splits;
   float m = -INFINITY, l = 0.f;
   if (lane < splits) {
@@ -779,7 +786,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
   int err = kvf_last_error();
   if (err || splits == 1) return err;
   hipLaunchKernelGGL(attn_split_combine_kernel, dim3(num_seqs, H), dim3(64), 0, s, part_acc,
-                     part_ml, seq_ids, cu_q, static_cast<bf16_t*>(out), H, d, splits, o_stride,
-                     n_seqs);
+                     part_ml, seq_ids, cu_q, ctx_lens, static_cast<bf16_t*>(out), H, d, splits,
+                     o_stride, n_seqs);
   return kvf_last_error();
 }

@@ -5,7 +5,7 @@
 //
 // Two kernels.  Many rows (a portion of a prompt): tiles of 64 x 64 outputs, every output summed
 // over k = 0..K-1 in that order by one thread.  Few rows (decode steps), where the product is
-// bound by reading W once: a wave owns four columns of W for all rows, its lanes walk K side by
+// bound by reading W once: a wave owns one to four columns of W for all rows, its lanes walk K side by
 // side with 16-byte loads (a wave reads 1 KB of a row of W at a time, several such loads in
 // flight), every lane keeps a partial sum per output and the 64 partial sums are added in a fixed
 // tree at the end.  Within either kernel a row's result does not depend on the number of rows, on

@@ -655,6 +655,31 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
     assert (got[[0, 2, 3, 5]] == 5.0).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_decode_in_cuts_clears_the_rows_of_empty_sequences(dtype):
+    """A captured batch is padded with sequences that hold nothing.  With the key range in cuts
+    their rows have no partial results; the merge must not read the workspace for them (it holds
+    whatever an earlier step left, NaNs here) and gives them zeros."""
+    H, KV, d, bs, splits = 8, 2, 64, 16, 4
+    seq_lens = [70, 1, 600]
+    paged = Paged(seq_lens, KV, d, bs, dtype, seed=3)
+    table = torch.cat([paged.table, torch.full((2, paged.table.shape[1]), -1, dtype=torch.int32)])
+    n = 5
+    g = torch.Generator().manual_seed(4)
+    buf = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    ctx = torch.tensor(seq_lens + [0, 0], dtype=torch.int32)
+    cu = torch.arange(n + 1, dtype=torch.int32)
+    scale = 1 / math.sqrt(d)
+    want = attn_reference(paged, buf[:3, :H * d].reshape(3, H, d), seq_lens, [1, 1, 1], scale, None)
+    ws = (torch.full((n * H * splits * d,), float("nan"), device=DEV),
+          torch.full((n * H * splits * 2,), float("nan"), device=DEV))
+    out = torch.full((n, H * d), 7.0, dtype=dtype, device=DEV)
+    ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), table.to(DEV), None, n, cu.to(DEV),
+                      ctx.to(DEV), out, H, KV, d, scale, 0, splits, ws, token_is_seq=True)
+    torch.testing.assert_close(out[:3].float().cpu(), want.reshape(3, H * d), **tol(dtype))
+    assert bool((out[3:] == 0).all())
+
+
 @pytest.mark.parametrize("slope", [0.12, 0.3, -0.2])
 def test_attn_scores_that_keep_rising_or_falling(slope):
     """Scores that grow (or shrink) steadily with the key's position, by less and by more per key
