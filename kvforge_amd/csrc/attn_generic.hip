@@ -6,7 +6,8 @@
 // kv head also share every K/V tile the workgroup loads.  Keys are walked in tiles aligned
 // to multiples of the tile size from position 0, with a running maximum, sum and accumulator
 // per row (all fp32).  Key j is visible to the query at position p iff j <= p, j < context
-// length and, with a window w > 0, j > p - w.  Scores are scaled after the dot product.
+// length and, with a window w > 0, j > p - w.  Scores are scaled after the dot product; with
+// `slopes` (one number per q head) slopes[h] * (j - p) is added to them, a bias by distance.
 //
 // K pages are [num_blocks, KV, block_size, d], V pages are transposed [num_blocks, KV, d,
 // block_size]; a key whose page entry is negative or out of range contributes nothing.
@@ -20,6 +21,7 @@ struct AttnArgs {
   int tiles_per_seq;  // 0: `work` holds (sequence, tile, tile or -1) rows; > 0: `work` lists sequences (or
                       // is null for 0, 1, 2, ...) and each takes this many tiles
   float scale;
+  const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
 };
 
 template <typename T, int DMAX, int BKEYS>
@@ -71,6 +73,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
   const int my_row = r0 + r;
   const bool row_ok = my_row < rows_total;
   const int my_pos = start + (row_ok ? my_row / G : 0);
+  const float slope = a.slopes && row_ok ? a.slopes[kvh * G + my_row % G] : 0.f;
   const int pos_min = start + r0 / G;
   int last_row = r0 + ROWS - 1;
   if (last_row >= rows_total) last_row = rows_total - 1;
@@ -121,7 +124,7 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
       const int j = t0 + c16 + 16 * jj;
       bool vis = row_ok && j <= my_pos && j < ctx;
       if (a.window > 0) vis = vis && (j > my_pos - a.window);
-      s[jj] = vis ? s[jj] * a.scale : -INFINITY;
+      s[jj] = vis ? fmaf(slope, static_cast<float>(j - my_pos), s[jj] * a.scale) : -INFINITY;
       tmax = fmaxf(tmax, s[jj]);
     }
 #pragma unroll
@@ -212,6 +215,7 @@ constexpr int DEC_WAVES = 4, DEC_KEYS = 64;
 struct DecodeArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs, splits;
   float scale;
+  const float* slopes;  // as in AttnArgs
 };
 
 // GT: heads of the group handled together (a power of two, at most 8; a larger group is taken
@@ -254,9 +258,10 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
   }
   __syncthreads();
 
-  float m_run[GT], l_run[GT], acc[GT][DQ];
+  float m_run[GT], l_run[GT], acc[GT][DQ], slope[GT];
 #pragma unroll
   for (int g = 0; g < GT; ++g) {
+    slope[g] = a.slopes && g0 + g < G ? a.slopes[kvh * G + g0 + g] : 0.f;
     m_run[g] = -INFINITY;
     l_run[g] = 0.f;
 #pragma unroll
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
     float corr[GT];
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
-      const float sc = (vis && page >= 0) ? s[g] * a.scale : -INFINITY;
+      const float sc = (vis && page >= 0) ? fmaf(slope[g], static_cast<float>(j - pos), s[g] * a.scale) : -INFINITY;
       const float m_new = fmaxf(m_run[g], wave_max(sc));
       float p = 0.f;
       corr[g] = 1.f;
@@ -473,13 +478,14 @@ KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_p
                                        void* out, float* part_acc, float* part_ml, int num_seqs,
                                        int H, int KV, int d, int block_size, int num_blocks,
                                        int table_stride, int q_stride, int o_stride, int window,
-                                       int n_seqs, int splits, float scale, hipStream_t s) {
+                                       int n_seqs, int splits, float scale, const float* slopes,
+                                       hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
       (splits > 1 && (!part_acc || !part_ml)) || block_size <= 0)
     return static_cast<int>(hipErrorInvalidValue);
   DecodeArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-               splits, scale};
+               splits, scale, slopes};
   if (dtype == 0)
     return launch_decode<float>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
                                 part_acc, part_ml, num_seqs, a, s);
@@ -498,12 +504,12 @@ KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, c
                                 const int* work, int num_work, int tiles_per_seq, void* out, int H,
                                 int KV, int d, int block_size, int num_blocks, int table_stride,
                                 int q_stride, int o_stride, int window, int n_seqs, float scale,
-                                hipStream_t s) {
+                                const float* slopes, hipStream_t s) {
   if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || tiles_per_seq < 0 ||
       (tiles_per_seq == 0 && !work))
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             tiles_per_seq, scale};
+             tiles_per_seq, scale, slopes};
   num_work *= tiles_per_seq > 0 ? tiles_per_seq : 2;
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);

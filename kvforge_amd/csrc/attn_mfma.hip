@@ -19,6 +19,8 @@
 //   operand by a rounding to bf16 alone; softmax itself is fp32.
 // Key j is visible to a query at position p iff j <= p, j < context length and, with a window
 // w > 0, j > p - w.  Scores are scaled after the dot product.
+// With `slopes` (one number per q head) a score also gets slopes[h] * (j - p), a bias by distance;
+// the kernels are instantiated with and without it, so that attention without it pays nothing.
 // The softmax reference of a row (what is subtracted before exp) is raised only when some score
 // of the wave exceeds it by more than LAZY (in log2 units): exp(s - ref) then stays below
 // 2^LAZY, sums and accumulators need no rescaling in most blocks, and the result is the same
@@ -59,6 +61,7 @@ struct MArgs {
   int H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits;
   float scale;
   unsigned bs_magic;  // floor(2^32 / bs) + 1: key / bs == mulhi(key, bs_magic) while key * bs < 2^32
+  const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
 };
 
 // Position of a key in its page table: (page table entry, slot in the page)
@@ -155,16 +158,21 @@ template <int RT> struct Rows {
   int tok[RT], head[RT];
   int first[RT];       // first visible key of the row
   unsigned span[RT];   // visible keys are first .. first + span; a row that is none has first < 0
+  int pos[RT];         // the row's own position; with slope2, only for kernels with BIAS
+  float slope2[RT];    // the head's slope in log2 units
 };
 
 // One key block for the row tiles of a wave: scores, lazy softmax update, P * V.
 // References live in log2 units: scale2 = scale * log2(e) > 0 is applied inside the exponent.
-template <int DT, int RT>
+// BIAS: a score also gets its head's slope times the key's distance from the row's position;
+// the scores are then brought to log2 units before the maximum is taken.
+template <int DT, int RT, bool BIAS>
 __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2], const bf16x8 (&vf)[DT],
                                              const bf16x8 (&qf)[RT][(DT + 1) / 2], const Rows<RT>& rows,
-                                             int kb, int kg, bool edge, float scale2, float (&m_ref)[RT], float (&l_run)[RT],
+                                             int kb, int kg, bool edge, float scale_log2, float (&m_ref)[RT], float (&l_run)[RT],
                                              f32x4 (&acc)[RT][DT]) {
   constexpr int DC = (DT + 1) / 2;
+  const float scale2 = BIAS ? 1.f : scale_log2;
   f32x4 s[RT][2];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -187,6 +195,17 @@ __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2]
           const bool vis = static_cast<unsigned>(key - rows.first[rt]) <= rows.span[rt];
           s[rt][t][r] = vis ? s[rt][t][r] : -INFINITY;
         }
+  }
+  if constexpr (BIAS) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const float at0 = rows.slope2[rt] * static_cast<float>(kb + 8 * kg - rows.pos[rt]);
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          s[rt][t][r] = fmaf(s[rt][t][r], scale_log2, fmaf(rows.slope2[rt], static_cast<float>(4 * t + r), at0));
+    }
   }
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
@@ -251,6 +270,8 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
       const int first = a.window > 0 && pos - a.window + 1 > 0 ? pos - a.window + 1 : 0;
       rows.first[rt] = rows.ok[rt] ? first : -1;
       rows.span[rt] = rows.ok[rt] ? static_cast<unsigned>(pos - first) : 0u;
+      rows.pos[rt] = pos;
+      rows.slope2[rt] = a.slopes && rows.ok[rt] ? a.slopes[rows.head[rt]] * LOG2E : 0.f;
     }
     if (seq_ok && (first_tile + rt) * 16 < rows_total) {
       int t_hi = ((first_tile + rt) * 16 + 15) / G;
@@ -270,7 +291,7 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
 // ------------------------------------------------------------------------------------ query runs
 // SHARE: the waves stage the fragments of each key block in LDS for each other; otherwise every
 // wave loads all of them itself.
-template <int DT, int RT, bool SHARE>
+template <int DT, int RT, bool SHARE, bool BIAS>
 __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -411,7 +432,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 #pragma unroll
         for (int t = 0; t < DT; ++t) vf[t] = as_frag(frag_lds[(buf * N_FRAG + N_K + t) * KVF_WAVE + lane]);
         const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-        block_update<DT, RT>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+        block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
       }
       if (more) put(buf ^ 1);
       __syncthreads();
@@ -440,7 +461,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 #pragma unroll
       for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(vr[t], vl));
       const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-      block_update<DT, RT>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+      block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
     }
   }
 
@@ -460,7 +481,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 // ------------------------------------------------------------------------- few rows, split keys
 // TWO: a wave holds the fragments of two blocks, loading one while it consumes the other.
 // NW: waves of the workgroup; more of them shorten each wave's walk over its cut of the keys.
-template <int DT, bool TWO, int NW>
+template <int DT, bool TWO, int NW, bool BIAS>
 __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -544,7 +565,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
 #pragma unroll
     for (int t = 0; t < DT; ++t) vf[t] = as_frag(keep_first(r.v[t], r.vl));
     const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
-    block_update<DT, 1>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
+    block_update<DT, 1, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
   };
   // Without a window the page lookups of the first blocks are asked for together with the
   // query and the context length, not after them: one round trip to memory less.
@@ -691,10 +712,16 @@ void launch_runs(dim3 grid, hipStream_t s, const void* q, const void* k_pages, c
   constexpr bool SHARE = runs_share(DT);
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
-  hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE>), grid, dim3(256), lds, s,
-                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
-                     static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
-                     static_cast<bf16_t*>(out), a);
+  if (a.slopes)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, true>), grid, dim3(256), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), a);
+  else
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false>), grid, dim3(256), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), a);
 }
 
 template <int DT, int NW>
@@ -702,10 +729,16 @@ void launch_split_waves(dim3 grid, hipStream_t s, const void* q, const void* k_p
                         const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
                         void* out, float* part_acc, float* part_ml, const MArgs& a) {
   const size_t lds = (static_cast<size_t>(NW) * DT * KVF_WAVE * 4 + NW * 16 * 2) * sizeof(float);
-  hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW>), grid, dim3(NW * KVF_WAVE), lds, s,
-                     static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
-                     static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
-                     static_cast<bf16_t*>(out), part_acc, part_ml, a);
+  if (a.slopes)
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, true>), grid, dim3(NW * KVF_WAVE), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), part_acc, part_ml, a);
+  else
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false>), grid, dim3(NW * KVF_WAVE), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), part_acc, part_ml, a);
 }
 
 int g_split_waves = 0;  // measurement aid: 4 or 8 waves per workgroup, 0 = by the grid
@@ -742,11 +775,12 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      const int* block_table, const int* cu_q, const int* ctx_lens,
                                      const int* work, int num_work, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
-                                     int window, int n_seqs, float scale, hipStream_t s) {
+                                     int window, int n_seqs, float scale, const float* slopes,
+                                     hipStream_t s) {
   if (num_work <= 0) return 0;
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale, magic_of(bs)};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale, magic_of(bs), slopes};
   const dim3 grid(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -765,12 +799,13 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     const int* ctx_lens, void* out, float* part_acc, float* part_ml,
                                     int num_seqs, int H, int KV, int d, int bs, int nb,
                                     int table_stride, int q_stride, int o_stride, int window,
-                                    int n_seqs, int splits, float scale, hipStream_t s) {
+                                    int n_seqs, int splits, float scale, const float* slopes,
+                                    hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs)};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs), slopes};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);

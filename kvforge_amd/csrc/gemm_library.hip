@@ -9,12 +9,13 @@
 //
 // Which algorithm: the first the library's heuristic names, except for row counts that come
 // back all the time (the powers of two from 32 to 512: the padded batches of captured decode
-// steps).  For those the heuristic's first CANDIDATES answers are timed once,
-// on the operands of the first call that may be repeated (not an accumulating one, not under
-// stream capture) and with the caches swept before every run, and the fastest is kept: a decode
-// step of 64 sequences at the 1B shape goes from 1.72 to 1.54 ms.  The engine's first call
-// of a shape is such a call (captures follow an eager step), so a shape's algorithm is settled
-// before its first result is handed out and equal calls give equal bits within a process.
+// steps).  For those the heuristic's first CANDIDATES answers are timed once, on the operands of
+// the shape's first call (into a C of the timing's own if the call adds into its C) and with the
+// caches swept before every run, and the fastest is kept: a decode step of 64 sequences at the
+// 1B shape goes from 1.72 to 1.54 ms.  A shape whose first call comes under stream capture cannot
+// be timed and keeps the heuristic's first answer for good (the engine's captures follow an
+// eager step, so its shapes are timed).  Either way a shape's algorithm is settled before its
+// first result is handed out, and equal calls give equal bits within a process.
 //
 // hipBLASLt counts in column-major matrices.  Row-major C[M, N] is column-major C^T[N, M] =
 // op(W) * A^T: the first operand is W as a K x N column-major matrix (leading dimension K),
@@ -197,10 +198,25 @@ KVF_EXPORT int kvf_gemm_library_bf16(const void* A, const void* W, void* C, int 
     const Key key{M, N, K, lda, ldc, out_f32 ? 1 : 0};
     auto it = dv.plans.find(key);
     if (it == dv.plans.end()) it = dv.plans.emplace(key, make_plan(dv, key)).first;
-    if (it->second.usable && !it->second.timed && !accumulate) {
+    if (it->second.usable && !it->second.timed) {
+      // The algorithm of a shape is settled before its first result is handed out and never
+      // changes afterwards, so equal calls give equal bits within a process.  A call that adds
+      // into C is timed on a C of its own; under capture nothing can be timed and the
+      // heuristic's first answer stays for good.
       hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-      if (hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone)
-        time_candidates(dv, it->second, A, W, C, s);
+      const bool eager = hipStreamIsCapturing(s, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusNone;
+      void* target = C;
+      void* own = nullptr;
+      if (eager && accumulate) {
+        if (hipMalloc(&own, static_cast<size_t>(M) * ldc * sizeof(float)) != hipSuccess) {
+          own = nullptr;
+          hipGetLastError();
+        }
+        target = own;
+      }
+      if (eager && target) time_candidates(dv, it->second, A, W, target, s);
+      it->second.timed = true;
+      if (own) hipFree(own);
     }
     plan = it->second;
     ws = dv.workspace;

@@ -170,13 +170,30 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, paired: bool = False) -> 
 
 
 # ------------------------------------------------------------------------------ rotary + cache
+NO_TABLE_LEN = 2**31 - 1
+
+
+def _rotary_tables(cos, sin, d: int, who: str):
+    """(cos pointer, sin pointer, rotary width, positions the tables cover).  Without tables
+    (both ``None``) nothing is rotated, the width is 0 and every position is covered."""
+    if cos is None and sin is None:
+        return None, None, 0, NO_TABLE_LEN
+    _check(cos, "cos", F32, (None, None))
+    _check(sin, "sin", F32, tuple(cos.shape))
+    table_len, half = cos.shape
+    if 2 * half > d or half <= 0:
+        raise KernelError(f"{who}: rotary width {2 * half} does not fit head_dim {d}")
+    return cos.data_ptr(), sin.data_ptr(), 2 * half, table_len
+
+
 def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
-                 cos: torch.Tensor, sin: torch.Tensor, block_table: torch.Tensor,
+                 cos: torch.Tensor | None, sin: torch.Tensor | None, block_table: torch.Tensor,
                  k_pages: torch.Tensor, v_pages: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, write_kv: bool = True) -> None:
     """Rotate q (in place) and k by the cos/sin rows of each token's position; write rotated k
     and v into the pages named by the token's sequence row of ``block_table``.  Rotary pairs
-    are neighbouring elements ``(2i, 2i + 1)`` of a head.  ``k_pages``:
+    are neighbouring elements ``(2i, 2i + 1)`` of a head; without tables (``None``) q and k stay
+    as they are and only the cache is written.  ``k_pages``:
     ``[num_blocks, KV, block_size, d]``; ``v_pages`` transposed: ``[num_blocks, KV, d, block_size]``."""
     n = qkv.shape[0]
     H, KV, d = num_heads, num_kv_heads, head_dim
@@ -185,12 +202,7 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
     _check(seq_of_token, "seq_of_token", I32, (None,))
     if positions.shape[0] < n or seq_of_token.shape[0] < n:
         raise KernelError("rope_kvwrite: positions / seq_of_token shorter than the batch")
-    _check(cos, "cos", F32, (None, None))
-    _check(sin, "sin", F32, tuple(cos.shape))
-    table_len, half = cos.shape
-    rot = 2 * half
-    if rot > d or rot <= 0:
-        raise KernelError(f"rope_kvwrite: rotary width {rot} does not fit head_dim {d}")
+    cos_p, sin_p, rot, table_len = _rotary_tables(cos, sin, d, "rope_kvwrite")
     _check(block_table, "block_table", I32, (None, None))
     n_seqs, stride = block_table.shape
     _check(k_pages, "k_pages", qkv.dtype, (None, KV, None, d))
@@ -198,8 +210,8 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
     _check(v_pages, "v_pages", qkv.dtype, (nb, KV, d, bs))
     f = _fn("elementwise", f"kvf_rope_kvwrite_{_suffix(qkv.dtype)}",
             [c_void_p] * 8 + [c_int] * 11 + [c_void_p])
-    _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(),
-          sin.data_ptr(), block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+    _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos_p,
+          sin_p, block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs, _stream()),
         "rope_kvwrite")
 
@@ -469,13 +481,13 @@ def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: flo
 
 
 def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positions: torch.Tensor,
-                  seq_of_token: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                  seq_of_token: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
                   block_table: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True,
                   rms_eps: float | None = None, a_owed: torch.Tensor | None = None) -> None:
     """Fused q/k/v projection: ``a @ w.T`` with rotary applied to q and k (neighbouring columns
     are pairs), rotated q stored to ``q_out [M, H*d]`` and rotated k and v written into the
-    pages.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; fp32, shape and
+    pages; without tables (``None``) nothing is rotated.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; fp32, shape and
     strides of ``a``): a sum still owed to ``a``; the projection is taken of ``a + a_owed``, and
     ``a`` itself is left as it is."""
     H, KV, d = num_heads, num_kv_heads, head_dim
@@ -496,11 +508,9 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     _check(seq_of_token, "seq_of_token", I32, (None,))
     if positions.shape[0] < m or seq_of_token.shape[0] < m:
         raise KernelError("gemm_qkv_rope: positions / seq_of_token shorter than the batch")
-    _check(cos, "cos", F32, (None, None))
-    _check(sin, "sin", F32, tuple(cos.shape))
-    table_len, half = cos.shape
-    if 2 * half > d or d % 4:
-        raise KernelError(f"gemm_qkv_rope: rotary width {2 * half} / head_dim {d} not supported")
+    cos_p, sin_p, rot, table_len = _rotary_tables(cos, sin, d, "gemm_qkv_rope")
+    if d % 4:
+        raise KernelError(f"gemm_qkv_rope: head_dim {d} not supported")
     _check(block_table, "block_table", I32, (None, None))
     _check(k_pages, "k_pages", BF16, (None, KV, None, d))
     nb, _, bs, _ = k_pages.shape
@@ -513,8 +523,8 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     wp, tiled = _w_args(w)
     _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, q_out.data_ptr(), m, k,
           a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d, float(rms_eps or 0.0),
-          a_owed.data_ptr() if a_owed is not None else None, positions.data_ptr(), seq_of_token.data_ptr(), cos.data_ptr(), sin.data_ptr(),
-          block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, 2 * half,
+          a_owed.data_ptr() if a_owed is not None else None, positions.data_ptr(), seq_of_token.data_ptr(), cos_p, sin_p,
+          block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, rot,
           table_len, bs, block_table.shape[1], nb, 1 if write_kv else 0, block_table.shape[0],
           _stream()), "gemm_qkv_rope")
 
@@ -617,6 +627,16 @@ def _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d
     return n_seqs
 
 
+def _slopes_ptr(slopes, H: int, like: torch.Tensor):
+    """Pointer to the per-head slopes of a bias by distance, or ``None`` for attention without."""
+    if slopes is None:
+        return None
+    _check(slopes, "slopes", F32, (H,))
+    if slopes.device != like.device:
+        raise KernelError("attention: slopes live on another device than q")
+    return slopes.data_ptr()
+
+
 def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
     """The MFMA attention kernels take bf16 and pages of a multiple of 8 tokens; everything else
     (the true 32-bit path above all) runs the vector-ALU kernel."""
@@ -633,39 +653,42 @@ def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int) ->
 def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
-                 head_dim: int, scale: float, window: int = 0) -> None:
+                 head_dim: int, scale: float, window: int = 0,
+                 slopes: torch.Tensor | None = None) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``prefill_rows_per_item(...)`` of them, and the items of one row are taken by
     one workgroup in turn (pair an early item with a late one).  ``v_pages`` are transposed:
-    ``[num_blocks, KV, head_dim, block_size]``."""
+    ``[num_blocks, KV, head_dim, block_size]``.  ``slopes``: fp32 ``[H]``; the score of key ``j``
+    for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     _check(work, "work", I32, (None, 3))
+    sl = _slopes_ptr(slopes, H, q)
     nb, _, bs, _ = k_pages.shape
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p])
+                [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
               cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], out.data_ptr(),
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window),
-              n_seqs, float(scale), _stream()), "attn_mfma_prefill")
+              n_seqs, float(scale), sl, _stream()), "attn_mfma_prefill")
         return
     _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, work.shape[0], 0, out,
-                  H, KV, d, scale, window, n_seqs)
+                  H, KV, d, scale, window, n_seqs, sl)
 
 
 def _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, tiles_per_seq,
-                  out, H, KV, d, scale, window, n_seqs) -> None:
+                  out, H, KV, d, scale, window, n_seqs, slopes_ptr=None) -> None:
     nb, _, bs, _ = k_pages.shape
     f = _fn("attn_generic", "kvf_attn_generic",
             [c_int] + [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 10
-            + [c_float, c_void_p])
+            + [c_float, c_void_p, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(),
           work.data_ptr() if work is not None else None, num_work, tiles_per_seq, out.data_ptr(),
           H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs,
-          float(scale), _stream()), "attn_generic")
+          float(scale), slopes_ptr, _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -673,15 +696,17 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 cu_q: torch.Tensor, ctx_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
-                token_is_seq: bool = False) -> None:
+                token_is_seq: bool = False, slopes: torch.Tensor | None = None) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
     (``num_seqs * H * splits * d``) and fp32 (max, sum) pairs (``num_seqs * H * splits * 2``).
     ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
-    single tokens), which spares the matrix-core kernel a dependent load."""
+    single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
+    ``attn_prefill``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
+    sl = _slopes_ptr(slopes, H, q)
     if token_is_seq and seq_ids is not None:
         raise KernelError("attn_decode: token_is_seq is for batches where every sequence decodes")
     if seq_ids is not None:
@@ -704,23 +729,23 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
             raise KernelError("attn_decode: workspace too small")
     if not attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_generic", "kvf_attn_generic_decode",
-                [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+                [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p, c_void_p])
         _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
               block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
               None if token_is_seq else cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
               pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
               num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
-              int(window), n_seqs, int(splits), float(scale), _stream()), "attn_generic_decode")
+              int(window), n_seqs, int(splits), float(scale), sl, _stream()), "attn_generic_decode")
         return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
-            [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p])
+            [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
           seq_ids.data_ptr() if seq_ids is not None else None,
           None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
           block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs, int(splits),
-          float(scale), _stream()), "attn_mfma_decode")
+          float(scale), sl, _stream()), "attn_mfma_decode")
 
 
 # ------------------------------------------------------------------------------ sampling

@@ -72,14 +72,18 @@ def prefill_work_rows(q_lens, prefill_seqs, group_size: int, rows_per_item: int)
 
 @register_mixer("attention")
 class PagedAttention(Mixer):
-    """``window``: ``None`` attends to every earlier position, ``w`` to the last ``w``."""
+    """``window``: ``None`` attends to every earlier position, ``w`` to the last ``w``.
+    ``rotary``: the rotation of q and k, or ``None`` for none.  ``score_slopes``: one number per
+    q head, or ``None``; the score of key ``j`` for a query at position ``p`` of head ``h`` then
+    gets ``score_slopes[h] * (j - p)`` added, a position encoding by distance that lives in the
+    scores instead of in q and k."""
 
     replayable = True
     settles_residual = True  # its norm kernel adds what is owed to the stream
 
     def __init__(self, prefix: str, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary: RotaryPositions | None, scale: float | None = None,
-                 window: int | None = None) -> None:
+                 window: int | None = None, score_slopes=None) -> None:
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         if head_dim % 16 or head_dim > 256:
@@ -90,6 +94,10 @@ class PagedAttention(Mixer):
         self.rotary = rotary
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         self.window = int(window) if window else None
+        self.score_slopes = None if score_slopes is None else [float(v) for v in score_slopes]
+        if self.score_slopes is not None and len(self.score_slopes) != self.H:
+            raise ValueError(f"score_slopes needs one number per q head ({self.H}), got {len(self.score_slopes)}")
+        self.slopes: torch.Tensor | None = None
         self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -118,6 +126,8 @@ class PagedAttention(Mixer):
         self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
         self.w_o = tensors[self._name("o_proj.weight")]
         self.norm_eps = None
+        if self.score_slopes is not None:
+            self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=self.w_o.device)
 
     def pair_permutation(self) -> torch.Tensor:
         """``perm[new] = old`` within a head: new elements 2i and 2i+1 are the checkpoint's
@@ -182,19 +192,6 @@ class PagedAttention(Mixer):
             step.scratch[key] = work
         return work
 
-    @staticmethod
-    def _no_rotation(step) -> tuple[torch.Tensor, torch.Tensor]:
-        """cos/sin tables of a rotation by zero, for attention without rotary positions: one
-        pair per head is "rotated" by the identity."""
-        tables = step.scratch.get("attention.no_rotation")
-        if tables is None:
-            n = int(step.positions.shape[0]) if step.positions is not None else 1
-            length = max(step.max_position + 1, n, 1)
-            tables = (torch.ones(length, 1, dtype=torch.float32, device=step.device),
-                      torch.zeros(length, 1, dtype=torch.float32, device=step.device))
-            step.scratch["attention.no_rotation"] = tables
-        return tables
-
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations, or (after ``absorb_norm``) the fp32 residual stream."""
         n = x.shape[0]
@@ -202,7 +199,7 @@ class PagedAttention(Mixer):
         ws = step.ws
         act = step.act_dtype
         table = step.block_tables[layer.group]
-        cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else self._no_rotation(step)
+        cos, sin = (self.rotary.cos, self.rotary.sin) if self.rotary is not None else (None, None)
         rms = self.norm_eps
         owed = None
         if rms is not None and not ops.bf16_kernel_takes(x, self.w_qkv, True):
@@ -239,7 +236,7 @@ class PagedAttention(Mixer):
         work = self._prefill_work(step, ops.prefill_rows_per_item(act, d, bs))
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
-                             work, out, H, KV, d, self.scale, window)
+                             work, out, H, KV, d, self.scale, window, self.slopes)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -249,5 +246,6 @@ class PagedAttention(Mixer):
             ops.attn_decode(qkv, layer.k_pages, layer.v_pages, table, step.decode_seq_ids,
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,
-                            token_is_seq=step.decode_seq_ids is None and work is None)
+                            token_is_seq=step.decode_seq_ids is None and work is None,
+                            slopes=self.slopes)
         add_product(step, out, self.w_o, residual, owed=owed)

@@ -454,6 +454,52 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
         assert all(torch.equal(x1, x2) for x1, x2 in zip(*got))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 40, 8), (32, 8, 64, 16)])
+@pytest.mark.parametrize("m", [1, 7, 48])
+def test_cache_write_without_rotation(dtype, H, KV, d, bs, m):
+    """Without rotary tables q and k stay as they are and only the cache is written, at any
+    position the block table covers: there is no table whose length could bound it.  Both the
+    kernel of its own and, in bf16, the projection that carries the write."""
+    g = torch.Generator().manual_seed(m + d)
+    width = (H + 2 * KV) * d
+    table = torch.randperm(300, generator=g)[:2 * 140].reshape(2, 140).to(torch.int32)
+    positions = (torch.randperm(140 * bs, generator=g)[:m]).to(torch.int32)        # far beyond any prompt here
+    seq_of = torch.randint(0, 2, (m,), generator=g, dtype=torch.int32)
+    args = (positions.to(DEV), seq_of.to(DEV), None, None, table.to(DEV))
+
+    def expect(qkv):
+        kp = torch.zeros(300, KV, bs, d, dtype=dtype)
+        vp = torch.zeros(300, KV, d, bs, dtype=dtype)
+        for i in range(m):
+            page, off = int(table[seq_of[i], positions[i] // bs]), int(positions[i]) % bs
+            kp[page, :, off] = qkv[i, H * d:(H + KV) * d].view(KV, d)
+            vp[page, :, :, off] = qkv[i, (H + KV) * d:].view(KV, d)
+        return kp, vp
+
+    qkv = torch.randn(m, width, generator=g).to(dtype)
+    on_dev = qkv.to(DEV)
+    kp = torch.zeros(300, KV, bs, d, dtype=dtype, device=DEV)
+    vp = torch.zeros(300, KV, d, bs, dtype=dtype, device=DEV)
+    ops().rope_kvwrite(on_dev, *args, kp, vp, H, KV, d)
+    want_k, want_v = expect(qkv)
+    assert torch.equal(on_dev.cpu(), qkv) and torch.equal(kp.cpu(), want_k) and torch.equal(vp.cpu(), want_v)
+    if dtype == torch.bfloat16 and d % 4 == 0:
+        k = 96
+        a = torch.randn(m, k, generator=g).to(dtype).to(DEV)
+        w = (torch.randn(width, k, generator=g) / 6).to(dtype).to(DEV)
+        proj = torch.empty(m, width, dtype=dtype, device=DEV)
+        ops().gemm(a, w, proj)
+        kp2, vp2, q2 = torch.zeros_like(kp), torch.zeros_like(vp), torch.empty(m, H * d, dtype=dtype, device=DEV)
+        ops().gemm_qkv_rope(a, w, q2, *args, kp2, vp2, H, KV, d)
+        want_k, want_v = expect(proj.cpu())
+        # the same kernel computes both up to SKINNY_MAX_M rows: the same bits; beyond, the plain
+        # product is the library's, with another order of sums
+        t = dict(atol=0, rtol=0) if m <= ops().SKINNY_MAX_M else dict(atol=2e-2, rtol=2e-2)
+        for got, want in ((q2, proj[:, :H * d]), (kp2, want_k), (vp2, want_v)):
+            torch.testing.assert_close(got.float().cpu(), want.float().cpu(), **t)
+
+
 @pytest.mark.parametrize("m", [5, 40])
 def test_gemm_rows_off_a_16_byte_boundary_take_the_plain_kernel(m):
     """Rows that start two bytes past a 16-byte boundary cannot be read 16 bytes at a time: neither
@@ -678,6 +724,83 @@ def test_attn_decode_in_cuts_clears_the_rows_of_empty_sequences(dtype):
                       ctx.to(DEV), out, H, KV, d, scale, 0, splits, ws, token_is_seq=True)
     torch.testing.assert_close(out[:3].float().cpu(), want.reshape(3, H * d), **tol(dtype))
     assert bool((out[3:] == 0).all())
+
+
+def attn_reference_with_slopes(paged, q, seq_lens, q_lens, scale, window, slopes):
+    """Whole-sequence attention in which the score of key ``j`` for the query at position ``p``
+    of head ``h`` is ``scale * q.k + slopes[h] * (j - p)``; written out row by row."""
+    outs, off = [], 0
+    for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
+        k, v = paged.keys[s].double(), paged.values[s].double()
+        G = q.shape[1] // k.shape[1]
+        out = torch.zeros(ql, q.shape[1], q.shape[2], dtype=torch.float64)
+        for i in range(ql):
+            p = n - ql + i
+            first = max(0, p - window + 1) if window else 0
+            j = torch.arange(first, p + 1)
+            for h in range(q.shape[1]):
+                sc = (k[first:p + 1, h // G] @ q[off + i, h].double()) * scale + float(slopes[h]) * (j - p).double()
+                out[i, h] = torch.softmax(sc, 0) @ v[first:p + 1, h // G]
+        outs.append(out)
+        off += ql
+    return torch.cat(outs).float()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16), (8, 2, 128, 16),
+                                        (32, 8, 64, 16), (20, 1, 16, 8), (4, 2, 32, 6)])
+@pytest.mark.parametrize("window", [0, 11])
+def test_attn_with_a_bias_by_distance(dtype, H, KV, d, bs, window):
+    """Slopes of both signs and of different size per head, for query runs and for single tokens
+    with the key range whole and in cuts.  A slope of the wrong sign, or one taken from another
+    head, moves the weight to the other end of the context."""
+    slopes = torch.tensor([(-1) ** h * 0.04 * (1 + h % 5) for h in range(H)], dtype=torch.float32)
+    scale = 1 / math.sqrt(d)
+    g = torch.Generator().manual_seed(d + H)
+    # query runs
+    seq_lens, q_lens = [12, 30, 5, 200], [4, 7, 5, 67]
+    paged = Paged(seq_lens, KV, d, bs, dtype, seed=d)
+    n = sum(q_lens)
+    buf = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    q = buf[:, :H * d].reshape(n, H, d)
+    cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+    ctx = torch.tensor(seq_lens, dtype=torch.int32)
+    out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
+    dev = (buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV))
+    ops().attn_prefill(*dev, cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV, dtype, d, bs).to(DEV),
+                       out, H, KV, d, scale, window, slopes=slopes.to(DEV))
+    want = attn_reference_with_slopes(paged, q.float(), seq_lens, q_lens, scale, window, slopes).reshape(n, H * d)
+    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    plain_out = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
+    assert (want - plain_out).abs().max() > 0.1          # the bias is no detail here
+    # single tokens
+    seq_lens = [7, 13, 1, 20, 300, 64]
+    paged = Paged(seq_lens, KV, d, bs, dtype, seed=d + 1)
+    n = len(seq_lens)
+    buf = torch.randn(n, (H + 2 * KV) * d, generator=g).to(dtype)
+    q = buf[:, :H * d].reshape(n, H, d)
+    cu = torch.arange(n + 1, dtype=torch.int32)
+    ctx = torch.tensor(seq_lens, dtype=torch.int32)
+    want = attn_reference_with_slopes(paged, q.float(), seq_lens, [1] * n, scale, window, slopes).reshape(n, H * d)
+    dev = (buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV))
+    for splits in (1, 3):
+        ws = (torch.empty(n * H * splits * d, device=DEV), torch.empty(n * H * splits * 2, device=DEV))
+        out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
+        ops().attn_decode(*dev, None, n, cu.to(DEV), ctx.to(DEV), out, H, KV, d, scale, window, splits, ws,
+                          slopes=slopes.to(DEV))
+        torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+
+
+def test_attn_slopes_are_checked():
+    H, KV, d, bs = 4, 2, 16, 4
+    paged = Paged([9], KV, d, bs, torch.float32)
+    buf = torch.randn(1, (H + 2 * KV) * d).to(DEV)
+    args = (buf, paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, 1,
+            torch.arange(2, dtype=torch.int32, device=DEV), torch.tensor([9], dtype=torch.int32, device=DEV),
+            torch.zeros(1, H * d, device=DEV), H, KV, d, 0.25)
+    for bad in (torch.zeros(H - 1, device=DEV), torch.zeros(H, dtype=torch.bfloat16, device=DEV), torch.zeros(H)):
+        with pytest.raises(Exception, match="slopes"):
+            ops().attn_decode(*args, slopes=bad)
 
 
 @pytest.mark.parametrize("slope", [0.12, 0.3, -0.2])
