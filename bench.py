@@ -291,6 +291,46 @@ def long_8b_points(batch=16, prompt_len=32768, new_tokens=128, warmup=8):
     return out
 
 
+def products_run(cfg, rows, repeats=6):
+    """The four matrix products of one layer alone, ``rows`` rows of bf16 activations each over
+    ``repeats`` copies of its weight in turn (so that no copy is found in a cache), through the
+    same entry points the parts use: microseconds per product.  For profiles and counters of a
+    single kernel."""
+    import torch
+    from kvforge_amd.kernels import ops
+    h, H, KV, d, I = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
+                      cfg["head_dim"], cfg["intermediate_size"])
+    dev, bf = "cuda", torch.bfloat16
+    ops.library_ready(dev)
+    out = {}
+    for name, (n, k) in {"qkv": ((H + 2 * KV) * d, h), "o": (h, H * d), "gate_up": (2 * I, h), "down": (h, I)}.items():
+        ws = [ops.streamed((torch.randn(n, k, device=dev) * 0.02).to(bf)) for _ in range(repeats)]
+        a = (torch.randn(rows, k, device=dev)).to(bf)
+        stream = torch.zeros(rows, n, device=dev)
+        plain = torch.empty(rows, n, device=dev, dtype=bf)
+        gated = torch.empty(rows, n // 2, device=dev, dtype=bf)
+
+        def launch(w):
+            if name in ("o", "down"):
+                ops.gemm(a, w, stream, accumulate=True)
+            elif name == "gate_up" and ops.bf16_kernel_takes(a, w, False, True):
+                ops.gemm_fused(a, w, gated, silu_pairs=True)
+            else:
+                ops.gemm(a, w, plain)
+        for w in ws:
+            launch(w)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for w in ws:
+            launch(w)
+        e1.record()
+        torch.cuda.synchronize()
+        out[f"{name}_us"] = round(e0.elapsed_time(e1) * 1e3 / repeats, 2)
+        del ws
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -319,12 +359,14 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products"], default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill; "
                          "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
                          "prefill beside decode steps, --steps new tokens each; burst: the "
                          "workload of the reference's own serving benchmark (48 short requests "
-                         "at once, 16 sequences a step), for --preset small or any other")
+                         "at once, 16 sequences a step), for --preset small or any other; "
+                         "products: the four matrix products of a layer alone at --batch rows "
+                         "(launch to launch, so short ones show the host's time)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -344,6 +386,10 @@ def main() -> int:
     nums = model_numbers(cfg, layers_run)
     vocab = cfg["vocab_size"]
 
+    if args.phase == "products":
+        print(json.dumps({"phase": "products", "model": args.preset, "rows": args.batch, "dtype": "bfloat16",
+                          **products_run(cfg, args.batch)}))
+        return 0
     with tempfile.TemporaryDirectory(prefix="kvforge_bench_") as folder:
         kvforge_amd.write_random_model(folder, cfg, seed=0)
         if args.phase == "burst":
