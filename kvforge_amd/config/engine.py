@@ -30,7 +30,10 @@ def parse_dtype(name: "str | torch.dtype") -> torch.dtype:
 
 
 class SchedulingPolicy(str, Enum):
+    """The order of the line (src/tokenvault/config.py:16-18): by arrival, or by the request's
+    ``priority`` first (a smaller number is served sooner) and by arrival within one priority."""
     FCFS = "fcfs"
+    PRIORITY = "priority"
 
 
 @dataclass

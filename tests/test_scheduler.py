@@ -23,9 +23,9 @@ class Driver:
                                device_runs=device_runs)
         self.cache = cache
 
-    def add(self, rid, prompt_len, arrival, max_tokens=8, **params):
+    def add(self, rid, prompt_len, arrival, max_tokens=8, priority=0, **params):
         req = Request(rid, range(1, prompt_len + 1), SamplingParams(max_tokens=max_tokens, **params),
-                      arrival_time=arrival)
+                      arrival_time=arrival, priority=priority)
         self.sched.add_request(req)
         return req
 
@@ -45,6 +45,36 @@ class Driver:
 
 def shares(plan):
     return [(s.request.request_id, s.count) for s in plan.slices]
+
+
+def test_priority_policy_orders_the_line_by_priority_then_arrival():
+    """src/tokenvault/scheduler.py:85-88: with the priority policy a smaller priority is served
+    sooner, arrival decides within one priority; without it the priority is not looked at."""
+    from kvforge_amd.config.engine import SchedulingPolicy
+    for policy, want in ((SchedulingPolicy.PRIORITY, ["late-urgent", "early-urgent", "early"]),
+                         (SchedulingPolicy.FCFS, ["early", "early-urgent", "late-urgent"])):
+        d = Driver(max_num_seqs=3, policy=policy)
+        d.add("early", 4, 1.0, priority=5)
+        d.add("early-urgent", 4, 2.0, priority=1)
+        d.add("late-urgent", 4, 3.0, priority=0)
+        assert [s.request.request_id for s in d.plan().slices] == want
+
+
+def test_priority_policy_preempts_the_least_urgent_and_readmits_it_behind_the_urgent():
+    """When pages run out the last in line gives way (src/tokenvault/scheduler.py:178-190): under
+    the priority policy that is the least urgent request, however early it came, and it goes back
+    in line at its place, behind a more urgent request that arrived meanwhile."""
+    from kvforge_amd.config.engine import SchedulingPolicy
+    d = Driver(num_blocks=4, block_size=4, max_num_seqs=4, policy=SchedulingPolicy.PRIORITY)
+    d.add("bulk", 7, 1.0, priority=9, max_tokens=6)
+    d.add("urgent", 7, 2.0, priority=0, max_tokens=6)
+    d.step()                                   # both prompts: two pages each, the pool is full
+    d.step()                                   # token 8 of each still fits its second page
+    plan = d.plan()                            # token 9 needs a third page
+    assert [r.request_id for r in plan.preempted] == ["bulk"] and shares(plan) == [("urgent", 1)]
+    d.ran(plan)
+    d.add("urgent-2", 3, 5.0, priority=1, max_tokens=2)
+    assert [r.request_id for r in d.sched._waiting] == ["urgent-2", "bulk"]
 
 
 def test_admission_follows_arrival_and_stops_at_max_num_seqs():
