@@ -701,14 +701,17 @@ bool args_ok(int H, int KV, int d, int bs, int nb, int table_stride, float scale
 unsigned magic_of(int bs) { return static_cast<unsigned>((1ull << 32) / bs) + 1u; }
 
 // Row tiles per wave and LDS sharing by head size: what fits the registers and 64 KB of LDS.
-constexpr int runs_rt(int) { return 1; }  // paired items balance the work; one tile per wave keeps more workgroups in flight
+// One tile per wave keeps more workgroups in flight; two halve what a key block costs per row
+// (looking its pages up, staging it, the barrier) and pay when the work fills the chip anyway
+// (measured at 32 heads of size 64: 8,192 tokens 525 to 441 us; 2,048 tokens 57 to 55; four
+// prompts of 512, 19.9 to 20.7): the caller chooses by the rows it has.
+constexpr int runs_max_rt(int dt) { return dt <= 8 ? 2 : 1; }
 constexpr bool runs_share(int dt) { return dt <= 12; }
 
-template <int DT>
-void launch_runs(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
-                 const int* block_table, const int* work, const int* cu_q, const int* ctx_lens, void* out,
-                 const MArgs& a) {
-  constexpr int RT = runs_rt(DT);
+template <int DT, int RT>
+void launch_runs_rt(dim3 grid, hipStream_t s, const void* q, const void* k_pages, const void* vt_pages,
+                    const int* block_table, const int* work, const int* cu_q, const int* ctx_lens, void* out,
+                    const MArgs& a) {
   constexpr bool SHARE = runs_share(DT);
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
@@ -722,6 +725,19 @@ void launch_runs(dim3 grid, hipStream_t s, const void* q, const void* k_pages, c
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
+}
+
+template <int DT>
+void launch_runs(int row_tiles, dim3 grid, hipStream_t s, const void* q, const void* k_pages,
+                 const void* vt_pages, const int* block_table, const int* work, const int* cu_q,
+                 const int* ctx_lens, void* out, const MArgs& a) {
+  if constexpr (runs_max_rt(DT) >= 2) {
+    if (row_tiles == 2) {
+      launch_runs_rt<DT, 2>(grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a);
+      return;
+    }
+  }
+  launch_runs_rt<DT, 1>(grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a);
 }
 
 template <int DT, int NW>
@@ -764,27 +780,34 @@ void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, 
   X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 }  // namespace
 
-// Rows of a query run one workgroup takes: 4 waves x RT tiles x 16 rows.
+// Rows of a query run one workgroup takes with `row_tiles` (1 or 2) tiles per wave, where the
+// head size allows so many: 4 waves x tiles x 16 rows.
 // For measurements: waves per workgroup of the kernel for single tokens (4, 8; 0 = by the grid).
 KVF_EXPORT void kvf_attn_mfma_set_split_waves(int waves) { g_split_waves = waves; }
-KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d) { return WAVES * runs_rt(d / 16) * 16; }
+KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d, int row_tiles) {
+  const int most = d > 0 && d <= 128 ? 2 : 1;   // runs_max_rt(d / 16)
+  return WAVES * (row_tiles >= 2 ? most : 1) * 16;
+}
 
 // Query runs: `work` holds num_work rows (sequence, item, item or -1) where item i covers rows
-// [i * rows_per_item, (i + 1) * rows_per_item) of the sequence's qlen * H/KV rows per kv head.
+// [i * rows_per_item, (i + 1) * rows_per_item) of the sequence's qlen * H/KV rows per kv head;
+// rows_per_item is what kvf_attn_mfma_rows_per_item gave for one or two row tiles.
 KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const void* vt_pages,
                                      const int* block_table, const int* cu_q, const int* ctx_lens,
-                                     const int* work, int num_work, void* out, int H, int KV, int d,
+                                     const int* work, int num_work, int rows_per_item, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
                                      int window, int n_seqs, float scale, const float* slopes,
                                      hipStream_t s) {
   if (num_work <= 0) return 0;
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
+  const int row_tiles = rows_per_item / (WAVES * 16);
+  if (rows_per_item != kvf_attn_mfma_rows_per_item(d, row_tiles)) return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale, magic_of(bs), slopes};
   const dim3 grid(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
-  case DT: launch_runs<DT>(grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a); break;
+  case DT: launch_runs<DT>(row_tiles, grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a); break;
     KVF_EACH_DT(GO)
 #undef GO
   }

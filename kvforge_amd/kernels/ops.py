@@ -643,10 +643,12 @@ def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
     return dtype == BF16 and block_size % 8 == 0
 
 
-def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int) -> int:
-    """Rows of (query token, head in group) that one entry of a prefill work list covers."""
+def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int, row_tiles: int = 1) -> int:
+    """Rows of (query token, head in group) that one entry of a prefill work list covers.
+    ``row_tiles``: 1 or 2 tiles of 16 rows per wave of the matrix-core kernel (two where the head
+    size allows them; they pay when the work fills the chip anyway, see ``attn_mfma.hip``)."""
     if attention_on_matrix_cores(dtype, block_size):
-        return int(_fn("attn_mfma", "kvf_attn_mfma_rows_per_item", [c_int])(int(head_dim)))
+        return int(_fn("attn_mfma", "kvf_attn_mfma_rows_per_item", [c_int, c_int])(int(head_dim), int(row_tiles)))
     return 16
 
 
@@ -654,10 +656,11 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, window: int = 0,
-                 slopes: torch.Tensor | None = None) -> None:
+                 slopes: torch.Tensor | None = None, rows_per_item: int | None = None) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
-    an item covers ``prefill_rows_per_item(...)`` of them, and the items of one row are taken by
+    an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
+    were made; by default its answer for one row tile), and the items of one row are taken by
     one workgroup in turn (pair an early item with a late one).  ``v_pages`` are transposed:
     ``[num_blocks, KV, head_dim, block_size]``.  ``slopes``: fp32 ``[H]``; the score of key ``j``
     for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``."""
@@ -666,14 +669,18 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     _check(work, "work", I32, (None, 3))
     sl = _slopes_ptr(slopes, H, q)
     nb, _, bs, _ = k_pages.shape
+    if rows_per_item is None:
+        rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p, c_void_p])
+                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
-              cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], out.data_ptr(),
+              cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], int(rows_per_item), out.data_ptr(),
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window),
               n_seqs, float(scale), sl, _stream()), "attn_mfma_prefill")
         return
+    if rows_per_item != 16:
+        raise KernelError("attn_prefill: the vector-ALU kernel takes items of 16 rows")
     _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, work.shape[0], 0, out,
                   H, KV, d, scale, window, n_seqs, sl)
 

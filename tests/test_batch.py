@@ -48,6 +48,11 @@ def test_flat_varlen_batch_reference_vector():
     assert prefill_work_rows(step.q_lens, step.prefill_seqs, 2, 16) == [(0, 0, -1)]
     assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 16) == [(0, 0, 1)]
     assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 4) == [(0, 0, 4), (0, 1, 3), (0, 2, -1)]
+    # a run half as far into its sequence as it is long, or farther, is not paired: one item
+    # per workgroup, the last (longest walk) first; a run nearer the start stays in pairs
+    q_lens = [3, 3, 1]
+    assert prefill_work_rows(q_lens, [0, 1], 6, 4, start_pos=[2, 1, 9]) == \
+        [(0, 4, -1), (0, 3, -1), (0, 2, -1), (0, 1, -1), (0, 0, -1), (1, 0, 4), (1, 1, 3), (1, 2, -1)]
 
 
 def test_wanted_places_and_modes():

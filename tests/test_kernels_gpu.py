@@ -614,10 +614,10 @@ def attn_reference(paged, q, seq_lens, q_lens, scale, window):
     return torch.cat(outs)
 
 
-def prefill_work(q_lens, G, dtype=torch.float32, d=16, bs=4):
+def prefill_work(q_lens, G, dtype=torch.float32, d=16, bs=4, row_tiles=1):
     """Rows (sequence, item, item or -1): an early item paired with a late one, as the engine
     does; the odd one out of three is left alone."""
-    rows = ops().prefill_rows_per_item(dtype, d, bs)
+    rows = ops().prefill_rows_per_item(dtype, d, bs, row_tiles)
     work = []
     for s, ql in enumerate(q_lens):
         n = -(-ql * G // rows)
@@ -642,6 +642,7 @@ ATTN_CASES = [
                                         (32, 8, 64, 16), (20, 1, 16, 8)])
 @pytest.mark.parametrize("window", [0, 11])
 def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
+    """Items of one row tile per wave and, where the kernel has them, of two."""
     paged = Paged(seq_lens, KV, d, bs, dtype, seed=len(seq_lens) + d)
     g = torch.Generator().manual_seed(d)
     n = sum(q_lens)
@@ -652,11 +653,16 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
     ctx = torch.tensor(seq_lens, dtype=torch.int32)
     out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
     scale = 1 / math.sqrt(d)
-    ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
-                       cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV, dtype, d, bs).to(DEV), out,
-                       H, KV, d, scale, window)
     want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
-    torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+    sizes = sorted({ops().prefill_rows_per_item(dtype, d, bs, tiles) for tiles in (1, 2)})
+    assert sizes == ([64, 128] if dtype == torch.bfloat16 and bs % 8 == 0 and d <= 128 else
+                     [64] if dtype == torch.bfloat16 and bs % 8 == 0 else [16])
+    for row_tiles, per_item in enumerate(sizes, 1):
+        out.zero_()
+        ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),
+                           cu.to(DEV), ctx.to(DEV), prefill_work(q_lens, H // KV, dtype, d, bs, row_tiles).to(DEV),
+                           out, H, KV, d, scale, window, rows_per_item=per_item)
+        torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -112,10 +112,16 @@ def test_embedding_and_head_parts(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("bs", [4, 8])
 @pytest.mark.parametrize("H,KV,d,window", [(6, 2, 16, None), (3, 1, 48, 7), (4, 4, 32, None)])
-def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
+@pytest.mark.parametrize("small_chip", [False, True])
+def test_attention_part_over_portions(dtype, H, KV, d, window, bs, small_chip, monkeypatch):
     """The attention part alone: a sequence fed in three portions (the last a single token) beside
     a second whole sequence gives the plain whole-sequence attention block; q and k projections
-    are scaled so the scores are peaked."""
+    are scaled so the scores are peaked.  ``small_chip``: the part is told of a chip without any
+    compute unit, which any rows fill, so it takes its items of two row tiles per wave
+    where the kernel has them."""
+    from kvforge_amd.parts import attention
+    if small_chip:
+        monkeypatch.setattr(attention, "_compute_units", {i: 0 for i in range(torch.cuda.device_count())})
     hidden = 40
     rot = RotaryPositions(d, 1000.0)
     rot.prepare(64, DEV)
@@ -151,6 +157,9 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs):
         residual = torch.zeros(x.shape[0], hidden, device=DEV)
         part.forward(x, step, ls, residual)
         step.settle()  # with many rows the last product is left owed to the stream
+        made = [v for k, v in step.scratch.items() if k[0] == "attention.prefill_work"]
+        if made and dtype == torch.bfloat16 and bs % 8 == 0:
+            assert made[0][1] == (128 if small_chip else 64)
         off = 0
         for rid, a, b in portions:
             got[rid].append(residual[off:off + b - a].cpu())
