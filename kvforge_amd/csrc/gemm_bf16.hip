@@ -618,16 +618,44 @@ int launch_one(const void* A, const bf16_t* W, void* C, int M, int N, int K, int
   return kvf_last_error();
 }
 
-// How many 16-row groups of W a wave takes: more when A has several row tiles and W has rows to
-// spare (the grid must still fill the chip).
+// Compute units of the current device, asked once per device.
+int compute_units() {
+  static int known[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (known[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    known[dev] = n;
+  }
+  return known[dev];
+}
+
+// How many 16-row groups of W a wave takes when A has several row tiles.  With 17 to 64 rows the
+// product is bound by what every compute unit has to bring in through its L1, which keeps only
+// some fifty lines in flight: all rows of A for each of its workgroups, and their columns of W.
+// A wave that takes more groups shares A's rows among more columns, but leaves fewer
+// workgroups; the choice is the one with the least to fill per compute unit, in rounds of
+// workgroups over the chip (measured at 32 rows: [5120, 3072] 15.2 us with one group, 10.9 with
+// two; [28672, 4096] 62.8 with two, 53.3 with four).
 template <int MT, int AT, int EPI>
 int launch_nt(const void* A, const bf16_t* W, void* C, int M, int N, int K, int lda, int ldc,
               int m_base, float eps, int w_tiled, const Riders& rd, const RopeEpi& rp, hipStream_t s) {
   const int tiles = (N + 15) / 16;
-  if (MT >= 2 && MT <= 4 && !AT) {
-    if (MT == 4 && tiles >= 1024)
+  if constexpr (MT >= 2 && MT <= 4 && !AT) {
+    const int cus = compute_units(), rows = M - m_base < MT * 16 ? M - m_base : MT * 16;
+    int best = 1, least = 0x7fffffff;
+    for (int nt = 1; nt <= 4; nt *= 2) {
+      const int groups = (tiles + nt - 1) / nt;
+      const int fill = ((groups + cus - 1) / cus) * (rows + 16 * nt);
+      if (fill < least) {
+        least = fill;
+        best = nt;
+      }
+    }
+    if (best == 4)
       return launch_one<MT, 4, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
-    if (tiles >= 512)
+    if (best == 2)
       return launch_one<MT, 2, AT, EPI>(A, W, C, M, N, K, lda, ldc, m_base, eps, w_tiled, rd, rp, s);
   }
   if (MT == 1) {
