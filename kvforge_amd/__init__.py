@@ -29,6 +29,7 @@ _LAZY = {
     "StepEntry": "kvforge_amd.engine.batch",
     "Transformer": "kvforge_amd.models.transformer",
     "ByteTokenizer": "kvforge_amd.tokenizer",
+    "FileTokenizer": "kvforge_amd.tokenizer",
 }
 
 

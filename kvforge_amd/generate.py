@@ -31,7 +31,8 @@ def parse_args(argv: list[str] | None = None) -> argparse.Namespace:
                       help="comma-separated token ids; repeat for several prompts")
     what.add_argument("--prompt-file", default=None, help="one prompt of token ids per line")
     what.add_argument("--prompt", action="append", default=None,
-                      help="text, tokenised byte by byte (needs vocab_size >= 258)")
+                      help="text, tokenised by the model folder's tokenizer.json if it has one, "
+                           "else byte by byte (needs vocab_size >= 258)")
     p.add_argument("--max-tokens", type=int, default=64)
     p.add_argument("--temperature", type=float, default=0.0)
     p.add_argument("--top-k", type=int, default=0)
@@ -65,9 +66,9 @@ def main(argv: list[str] | None = None) -> int:
     from kvforge_amd.config.engine import CacheConfig, EngineConfig, SchedulerConfig
     from kvforge_amd.engine.engine import InferenceEngine
     from kvforge_amd.sampling.params import SamplingParams
-    from kvforge_amd.tokenizer import ByteTokenizer
+    from kvforge_amd.tokenizer import tokenizer_for
 
-    tokenizer = ByteTokenizer() if args.prompt else None
+    tokenizer = tokenizer_for(args.model) if args.prompt else None
     if args.prompt:
         prompts: list = list(args.prompt)
     elif args.prompt_file:

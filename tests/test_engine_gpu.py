@@ -658,6 +658,32 @@ def test_command_line(model_a, capsys):
     assert rec["stats"]["kv_cache"]["num_blocks"] == 32
 
 
+def test_command_line_with_text_and_the_folders_own_tokenizer(model_a, capsys, tmp_path):
+    """``--prompt`` goes through the model folder's tokenizer.json when it has one: the same
+    tokens as the ids given directly, and the output comes back as text."""
+    import json
+    import shutil
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    from kvforge_amd import generate
+    folder, oracle = model_a
+    mine = str(tmp_path / "with_tokenizer")
+    shutil.copytree(folder, mine)
+    words = ["<unk>"] + [f"w{i}" for i in range(1, 60)]
+    tok = tokenizers.Tokenizer(WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tok.pre_tokenizer = Whitespace()
+    tok.save(mine + "/tokenizer.json")
+    rc = generate.main(["--model", mine, "--prompt", "w5 w17 w3", "--max-tokens", "6", "--temperature", "0",
+                        "--block-size", "4", "--num-blocks", "32", "--ignore-eos", "--json"])
+    assert rc == 0
+    out = json.loads(capsys.readouterr().out.strip().splitlines()[-1])["outputs"][0]
+    assert out["prompt_token_ids"] == [5, 17, 3]
+    want, gaps = oracle.greedy([5, 17, 3], 6)
+    assert_greedy_equal(out["output_token_ids"], want, gaps)
+    assert out["text"] == tok.decode(out["output_token_ids"])
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_equals_eager_steps(model_b, dtype):
     """Decode steps replayed from captured HIP graphs give the tokens of the same steps launched
