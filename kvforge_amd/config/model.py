@@ -249,7 +249,3 @@ def read_config_json(folder_or_file: str) -> dict[str, Any]:
     if not isinstance(d, dict):
         raise ConfigError(f"{path} does not hold a JSON object")
     return d
-
-
-def config_field_names(cfg: ModelConfig) -> list[str]:
-    return [f.name for f in fields(cfg)]
