@@ -116,7 +116,11 @@ def test_llama3_scaling_mid_band_value_worked_by_hand():
     A blend that is linear in the wavelength instead (s = (64 - 32.4) / 48) gives 0.1442 and
     passes every bound, order and continuity check above.  The plain model and the engine's
     tables must both give the worked value; neighbours j = 1 (wavelength 14.27, kept) and j = 3
-    (73.58, divided by 4) pin the two thresholds' sides."""
+    (73.58, divided by 4) pin the two thresholds' sides.
+
+    Parity unpinned: the reference has no frequency scaling and nothing it ships holds a vector
+    of scaled frequencies, so the worked value follows from the rule as written above and from
+    no output of the reference."""
     from kvforge_amd.config.model import RopeScaling
     from kvforge_amd.parts.positions import scaled_inv_freq
     base = plain.rope_inv_freq(32, 500000.0)
