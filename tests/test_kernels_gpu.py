@@ -166,6 +166,34 @@ def test_gemm_bf16_mfma(m, n, k):
     torch.testing.assert_close(out2.double().cpu(), want, **t32)
 
 
+@pytest.mark.parametrize("m", [20, 32, 50, 64])
+@pytest.mark.parametrize("n,k", [(16400, 256), (5120, 96), (4104, 512), (40000, 64)])
+def test_gemm_bf16_rows_in_two_to_four_tiles_over_many_columns(m, n, k, monkeypatch):
+    """17 to 64 rows over weights with so many columns that a wave takes two or four groups of
+    16 of them (the choice follows the columns and the chip): every store, with columns that end
+    inside a group."""
+    monkeypatch.setattr(ops(), "SKINNY_MAX_M", 64)
+    monkeypatch.setattr(ops(), "is_library_product", lambda a, w: False)
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(DEV)
+    plain_w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16).to(DEV)
+    want = a.double().cpu() @ plain_w.double().cpu().T
+    res = torch.randn(m, n, generator=g)
+    for w in (plain_w, ops().StreamedWeight(plain_w)):
+        out, acc = torch.empty(m, n, device=DEV), res.clone().to(DEV)
+        outb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        gate = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
+        ops().gemm(a, w, out)
+        ops().gemm(a, w, outb)
+        ops().gemm(a, w, acc, accumulate=True)
+        ops().gemm_fused(a, w, gate, silu_pairs=True)
+        torch.testing.assert_close(out.double().cpu(), want, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(outb.double().cpu(), want, atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(acc.double().cpu(), res.double() + want, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(gate.double().cpu(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2],
+                                   atol=1e-2, rtol=1e-2)
+
+
 @pytest.mark.parametrize("m", [33, 64, 100, 257])
 @pytest.mark.parametrize("n,k", [(37, 96), (384, 176), (2048, 2048), (200, 8192), (3072, 64)])
 def test_gemm_of_many_rows_through_the_library_entry_point(m, n, k):
