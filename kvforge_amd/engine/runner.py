@@ -50,6 +50,11 @@ class ModelRunner:
         self.meta = MetaBuffers(max(max_num_batched_tokens, max_num_seqs), max_num_seqs,
                                 [width] * len(groups), self.device)
         self.ws = Workspace(self.device)
+        # The residual stream is where a captured step that ends in the head's greedy pick finds
+        # its first embeddings, written either by the step before it or by the host's embedding
+        # of a run's first tokens: one piece of memory for every step there will be, made at its
+        # full size now, so that no later, longer step makes the workspace move it.
+        self.ws.buf("residual", (self.meta.max_tokens, model.spec.embedding.hidden), torch.float32)
         self._windowed = [g.window is not None for g in groups]
         self.num_forward_passes = 0
         self.num_tokens_processed = 0

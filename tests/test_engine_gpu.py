@@ -641,6 +641,35 @@ def test_long_decoding(model_b):
             assert_greedy_equal(out.output_token_ids, want, gaps, margin)
 
 
+def test_captured_greedy_steps_after_the_workspace_has_grown(model_a):
+    """A captured step that ends in the head's greedy pick finds its first embeddings where the
+    step before left them, or where the host's embedding of a new run's first token put them:
+    both must be the memory the graph was recorded with, also after a long prompt has made the
+    workspace's buffers grow.  One request decodes alone (the graph is recorded while the buffers
+    are small), a long prompt passes through, and another request decodes alone through the
+    same graph."""
+    folder, oracle = model_a
+    greedy = SamplingParams(max_tokens=14, temperature=0.0)
+
+    def run(long_prompt_between):
+        engine = engine_for(folder, "bfloat16", num_blocks=128, max_num_seqs=4, max_num_batched_tokens=256)
+        assert engine.runner.use_graphs and engine.model.can_pick(1)
+        first = engine.generate([[5, 17, 3, 11, 2, 40]], greedy)[0].output_token_ids
+        tails = engine.runner.num_greedy_tails
+        assert tails > 0
+        if long_prompt_between:
+            engine.generate([prompts_for(256, 1, 9, 100, 100)[0]], SamplingParams(max_tokens=1, temperature=0.0))
+        second = engine.generate([[9, 8, 7, 6]], greedy)[0].output_token_ids    # no longer than the first
+        assert engine.runner.num_greedy_tails > tails and len(engine.runner.graphs) == 1
+        return first, second
+
+    # the same kernels either way: the same tokens, whatever passed through in between
+    assert run(True) == run(False)
+    for prompt, out in zip(([5, 17, 3, 11, 2, 40], [9, 8, 7, 6]), run(True)):
+        oracle.check_choices(prompt, out, 3e-2)
+        assert out != [prompt[-1]] * 14
+
+
 def test_command_line(model_a, capsys):
     from kvforge_amd import generate
     folder, oracle = model_a
