@@ -404,7 +404,7 @@ def test_gemm_fused_norm_and_gate(m, n, k):
 # the norm rides in the projection only for one tile of rows
 @pytest.mark.parametrize("m,rms", [(m, r) for m in (1, 9, 16, 23, 40, 64) for r in (False, True) if m <= 16 or not r])
 @pytest.mark.parametrize("H,KV,d,rot,bs", [(4, 2, 16, 16, 4), (3, 1, 32, 32, 8), (2, 2, 48, 32, 16),
-                                            (32, 8, 64, 64, 16)])
+                                            (32, 8, 64, 64, 16), (40, 8, 128, 128, 16)])
 def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     """The fused projection + rotary + cache write against projection (MFMA kernel), then the
     rotary/cache-write kernel: same q, same pages."""
