@@ -527,6 +527,51 @@ def test_random_traffic_gives_the_same_tokens_however_it_is_run(model_a, seed):
     assert saw_ahead > 0                                        # and runs are meant to be queued ahead
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_the_heads_greedy_pick_gives_the_tokens_of_logits_and_argmax(model_a, seed):
+    """Captured steps whose rows are all greedy end in the head's own kernel: no logits, the
+    next inputs and embeddings made there.  The product's sums are those of the kernel that
+    stores logits, so every token must be the one that the stored logits' largest entry names:
+    random traffic in bf16 (requests of random lengths arriving while others decode, long
+    prompts that make the workspace grow, token limits and stop tokens that cut runs short, a
+    pool that runs out) through an engine with the pick and one without it."""
+    folder, oracle = model_a
+    rng = random.Random(40 + seed)
+    n = 10
+    prompts = [prompts_for(256, 1, 300 + seed * 20 + i, lo, hi)[0]
+               for i, (lo, hi) in enumerate([(1, 12)] * 6 + [(60, 110)] * 2 + [(1, 30)] * 2)]
+    rng.shuffle(prompts)
+    params = [SamplingParams(max_tokens=rng.randint(1, 45), temperature=0.0,
+                             stop_token_ids=rng.sample(range(256), rng.choice([0, 0, 10])))
+              for _ in range(n)]
+    arrive = sorted(rng.randint(0, 14) for _ in range(n))
+
+    def run(with_pick):
+        engine = engine_for(folder, "bfloat16", block_size=4, num_blocks=80, max_num_seqs=4,
+                            max_num_batched_tokens=128, seed=5)
+        assert engine.runner._tail is not None
+        if not with_pick:
+            engine.runner._tail = None
+        ids, outs, step = {}, {}, 0
+        while len(ids) < n or engine.has_unfinished_requests():
+            for i in range(n):
+                if i not in ids and arrive[i] <= step:
+                    ids[i] = engine.add_request(prompts[i], params[i])
+            for o in engine.step():
+                outs[o.request_id] = o
+            step += 1
+            assert step < 2000
+        assert engine.cache.num_free_blocks == engine.cache.num_blocks
+        return [(outs[ids[i]].output_token_ids, outs[ids[i]].finish_reason) for i in range(n)], engine
+
+    want, plain_engine = run(False)
+    got, engine = run(True)
+    assert engine.runner.num_greedy_tails > 20 and plain_engine.runner.num_greedy_tails == 0
+    assert got == want
+    for i, (tokens, _) in enumerate(got):
+        oracle.check_choices(prompts[i], tokens, 3e-2)
+
+
 @pytest.mark.parametrize("use_graphs", [True, False])
 def test_an_id_used_again_brings_its_own_sampling_parameters(model_b, use_graphs):
     """Request "a" runs greedy to its end; then "a" again, alone, with a temperature, then once
