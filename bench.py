@@ -219,13 +219,14 @@ def prefill_flops(nums, n):
             + 2.0 * n * n * nums["attn_hd"] * nums["layers"])
 
 
-def fp32_points(folder, cfg, vocab, nums, steps=48, warmup=8):
-    """The 1B shape in true 32-bit: decode at batch 1 and 8, prefill of 2,048 tokens."""
+def fp32_points(cfg, vocab, nums, steps=48, warmup=8):
+    """The 1B shape in true 32-bit, weights drawn and held in 32-bit on the device: decode at
+    batch 1 and 8, prefill of 2,048 tokens."""
     import torch
     out = {}
     for b in (8, 1):
         need = b * (512 + steps + warmup + early_tokens(b, 512) + 32)
-        engine = build_engine(folder, "float32", b, max(need, PREFILL_TOKENS + 64))
+        engine = build_engine(cfg, "float32", b, max(need, PREFILL_TOKENS + 64))
         r = decode_run(engine, vocab, b, 512, steps, warmup)
         out[f"fp32_decode_b{b}"] = round(r["tok_s"], 1)
         out[f"fp32_decode_b{b}_ms"] = round(r["ms_per_step"], 4)
@@ -391,7 +392,7 @@ def main() -> int:
                           **products_run(cfg, args.batch)}))
         return 0
     with tempfile.TemporaryDirectory(prefix="kvforge_bench_") as folder:
-        kvforge_amd.write_random_model(folder, cfg, seed=0)
+        kvforge_amd.write_random_model(folder, cfg, seed=0, dtype=args.dtype)
         if args.phase == "burst":
             prompt_tokens, (dt, generated, summary, passes) = burst_run(folder, vocab, args.dtype,
                                                                         not args.no_graphs)
@@ -436,7 +437,7 @@ def main() -> int:
         more = {}
         if points and args.preset == "llama-1b" and layers_run == full_layers:
             chosen = set((args.only_points or "fp32,mixed_3b,long_8b").split(","))
-            for name, fn in (("fp32", lambda: fp32_points(folder, cfg, vocab, nums)),
+            for name, fn in (("fp32", lambda: fp32_points(cfg, vocab, nums)),
                              ("mixed_3b", mixed_3b_points), ("long_8b", long_8b_points)):
                 if name not in chosen:
                     continue

@@ -384,9 +384,10 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
     }
     const int head = kvh * G + g0 + g;
     if (a.splits == 1) {
-      if (ctx > 0)
-        Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * D + e,
-                       l > 0.f ? o / l : 0.f);
+      // a sequence without context (padding of a captured batch) gets zeros, as the merge
+      // kernel gives it: no row of the output keeps what an earlier step left there
+      Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * D + e,
+                     l > 0.f ? o / l : 0.f);
     } else {
       const size_t p = (static_cast<size_t>(slot) * a.H + head) * a.splits + cut;
       part_acc[p * D + e] = o;

@@ -626,6 +626,16 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     cw[w] = mw == -INFINITY ? 0.f : exp2f(mw - mm);
     ll += red_ml[(w * 16 + j16) * 2 + 1] * cw[w];
   }
+  if (a.splits == 1 && qlen == 1 && ctx <= 0) {
+    // a sequence without context (the padding of a captured batch): a row of zeros, as the merge
+    // of cuts gives it, so that no row of the output keeps what an earlier step left there
+    const int g = tile * 16 + j16;
+    if (g < G)
+      for (int t = wave; t < DT; t += NW)
+        *reinterpret_cast<uint2*>(out + static_cast<size_t>(q0) * a.o_stride + (kvh * G + g) * D + t * 16 +
+                                  4 * kg) = make_uint2(0u, 0u);
+    return;
+  }
   if (!rows.ok[0]) return;
   const int head = rows.head[0];
   const size_t slot = (static_cast<size_t>(entry) * a.H + head) * a.splits + blockIdx.z;

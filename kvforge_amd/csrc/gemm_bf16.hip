@@ -116,14 +116,22 @@ __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
 }
 
 // Results that other workgroups are going to read are stored past this XCD's L2 (an atomic store
-// at device scope is written through); before a ticket is taken they only have to be complete.
+// at device scope is written through); before a ticket is taken they have to be complete.
 // A device-scope release fence would also write the whole L2's dirty lines back, and thousands
-// of workgroups doing that made the head's product take 275 us instead of 90.
+// of workgroups doing that made the head's product take 275 us instead of 90.  What orders the
+// results before the ticket instead: every wave that published waits until its stores have been
+// acknowledged (the vector memory counter at zero: a written-through store is acknowledged from
+// where the device's other L2s read it), then comes the workgroup's barrier, and only then does
+// thread 0 add to the ticket.  A fence of workgroup scope alone would not do: it lets stores to
+// global memory stay in flight, since all waves of a workgroup share one L1.
 __device__ __forceinline__ void pick_publish(float* val, int* idx, size_t at, float v, int i) {
   __hip_atomic_store(val + at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __hip_atomic_store(idx + at, i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void pick_stores_done() { __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); }
+__device__ __forceinline__ void pick_stores_done() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 
 // The last arrival at counter `lane`: the best per row over the workgroups lane, lane + 64, ...
 // into the second level of the scratch ([16][PICK_LANES] behind the first).  All threads of the

@@ -428,6 +428,20 @@ __global__ void clear_ints_kernel(int* __restrict__ p, int n) {
   if (i < n) p[i] = 0;
 }
 
+// Compute units of the current device, asked of the runtime once per device; 0 if it does not say.
+int compute_units_of_current_device() {
+  static int units[MAX_DEVICES];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 0;
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (units[dev] <= 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    units[dev] = n;
+  }
+  return units[dev];
+}
+
 // The device address of `scratch` on the current device; null (and *code set) if the runtime
 // does not give it.
 int* scratch_on_current_device(hipError_t* code) {
@@ -464,7 +478,9 @@ KVF_EXPORT int kvf_sample_static(const float* logits, int ld, int rows, int V, c
   if (V <= 0 || ld < V) return static_cast<int>(hipErrorInvalidValue);
   // about one workgroup per compute unit, each with at least 4096 logits
   int splits = KVF_SAMPLE_STATIC_MAX_SPLITS;
-  if (splits > 256 / rows) splits = 256 / rows;
+  const int units = compute_units_of_current_device();
+  if (units <= 0) return static_cast<int>(hipErrorInvalidDevice);
+  if (splits > units / rows) splits = units / rows;
   if (splits > V / 4096) splits = V / 4096;
   if (splits < 1) splits = 1;
   int* work = nullptr;

@@ -49,6 +49,7 @@ class InferenceEngine:
                                    device_runs=self.runner.takes_runs)
         self.metrics = MetricsCollector()
         self._num_added = 0
+        self.stalled = False      # the last step found requests but nothing to plan
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -63,7 +64,8 @@ class InferenceEngine:
                     tokenizer: Any = None, seed: int | None = None,
                     on_device: bool = False) -> "InferenceEngine":
         """Random weights: ``model_config`` is a config.json dictionary or a preset name; the
-        model folder is written to a temporary place and loaded like any other.  With
+        model folder is written to a temporary place, stored in the engine's type (a float32
+        engine gets 32-bit weights), and loaded like any other.  With
         ``on_device`` the tensors are drawn on the GPU instead and no file is written (for
         models of many gigabytes; other numbers than the folder's for the same seed)."""
         from kvforge_amd.config.presets import preset_dict
@@ -75,7 +77,7 @@ class InferenceEngine:
                                             config.device)
             return cls(model, config, tokenizer)
         with tempfile.TemporaryDirectory(prefix="kvforge_amd_model_") as tmp:
-            write_random_model(tmp, d, config.seed if seed is None else seed)
+            write_random_model(tmp, d, config.seed if seed is None else seed, dtype=config.dtype)
             return cls.from_folder(tmp, config, tokenizer)
 
     # ------------------------------------------------------------------ requests in
@@ -134,6 +136,10 @@ class InferenceEngine:
         final: dict[str, RequestOutput] = {}
         while self.has_unfinished_requests() and len(final) < len(order):
             final.update((o.request_id, o) for o in self.step() if o.finished)
+            if self.stalled:
+                raise RuntimeError(
+                    f"nothing can be planned although {self.scheduler.num_waiting} request(s) "
+                    f"wait and {self.scheduler.num_running} run: the scheduler is stuck")
         return [final[rid] for rid in order if rid in final]
 
     # ------------------------------------------------------------------ one step
@@ -144,6 +150,10 @@ class InferenceEngine:
         queued = self.runner.queued_run_steps(
             [(r.request_id, r.computed) for r in self.scheduler.running])
         plan = self.scheduler.schedule(queued_steps=queued)
+        # A plan without tokens that took nobody's pages either changes nothing: the next one
+        # would be the same.  ``generate`` raises on it instead of asking for ever.
+        self.stalled = (plan.is_empty and not plan.preempted
+                        and self.scheduler.has_unfinished())
         if plan.is_empty:
             return []
         sampled = self._execute(plan)

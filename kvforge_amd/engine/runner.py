@@ -90,7 +90,7 @@ class ModelRunner:
         self._tail: DecodeTail | None = None
         if self.use_graphs and model.can_pick(1):
             self._tail = DecodeTail(self._sample_i[cap:2 * cap], self._run_ring, self._run_counter,
-                                    model.spec.embedding.table,
+                                    model.spec.embedding.pick_table(),
                                     ops.pick_workspace(16, model.config.vocab_size, self.device))
 
     @staticmethod

@@ -228,12 +228,22 @@ FUSED_EPILOGUE_MAX_M = 64
 _GEMM_BF16_ARGS = ([c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 6
                    + [c_float, c_void_p, c_void_p, c_void_p])
 # A product that is added to a narrow fp32 stream (few output columns, long K) has too few
-# workgroups to pull on the weights with all of the chip: with at most this many groups of 16
-# columns (half the compute units) and from this K on it is cut into two halves of K
+# workgroups to pull on the weights with all of the chip: with groups of 16 columns for at most
+# half the compute units and from this K on it is cut into two halves of K
 # (``k_halves_pay``).  The half that is left owed costs its consumers a second fp32 operand, so
 # wider streams lose more there than the product gains (measured at 3072 columns: 7% of the step).
-K_HALVES_MAX_GROUPS = 128
 K_HALVES_MIN_K = 4096
+_compute_units: dict[int, int] = {}
+
+
+def compute_units(device) -> int:
+    """Compute units of the device, asked of the device once."""
+    index = torch.device(device).index
+    if index is None:
+        index = torch.cuda.current_device()
+    if index not in _compute_units:
+        _compute_units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _compute_units[index]
 
 
 class StreamedWeight:
@@ -349,7 +359,7 @@ def k_halves_pay(a: torch.Tensor, w) -> bool:
     m, k = a.shape
     return (not is_library_product(a, w) and a.dtype == BF16 and plain_of(w).dtype == BF16
             and k % 8 == 0 and m <= 16 and k >= K_HALVES_MIN_K
-            and -(-w.shape[0] // 16) <= K_HALVES_MAX_GROUPS)
+            and -(-w.shape[0] // 16) <= compute_units(a.device) // 2)
 
 
 # The library's product is called through an entry point of our own: torch.mm costs 17 us of
@@ -800,7 +810,7 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor 
         if work.shape[0] < sample_work_size(r):
             raise KernelError("sample: work is smaller than sample_work_size(rows)")
         # about one workgroup per compute unit, each with at least 4096 logits
-        splits = max(1, min(GREEDY_SPLIT_MAX, 256 // r, v // 4096))
+        splits = max(1, min(GREEDY_SPLIT_MAX, compute_units(logits.device) // r, v // 4096))
     f = _fn("sampling", "kvf_sample",
             [c_void_p, c_int, c_int, c_int] + [c_void_p] * 5 + [c_int, c_void_p, c_void_p, c_int,
                                                                 c_void_p])

@@ -58,15 +58,19 @@ class Transformer:
         return model
 
     @classmethod
-    def from_random(cls, config, seed: int, dtype: torch.dtype, device: torch.device | str = "cuda"
-                    ) -> "Transformer":
+    def from_random(cls, config, seed: int, dtype: torch.dtype, device: torch.device | str = "cuda",
+                    drawn: "dict[str, torch.Tensor] | None" = None) -> "Transformer":
         """Random weights drawn on the device, no files (``config``: a config.json dictionary or
-        a typed configuration)."""
+        a typed configuration).  ``drawn``, if given, is filled with the tensors by checkpoint
+        name as they were drawn, for whoever wants to compute the same model another way."""
         from kvforge_amd.weights.random_init import load_random_weights
 
         cfg = registry.config_from_dict(config) if isinstance(config, dict) else config
         model = cls(registry.build_spec(cfg), dtype, device)
-        load_random_weights(model.spec, seed, dtype, device)
+        tensors = load_random_weights(model.spec, seed, dtype, device)
+        if drawn is not None:
+            drawn.update(tensors)
+        del tensors
         model._seal()
         return model
 
@@ -134,15 +138,13 @@ class Transformer:
     # ------------------------------------------------------------------ forward
     def can_pick(self, rows: int) -> bool:
         """Whether a decode step of ``rows`` sequences can end in the head's greedy pick
-        (``forward(step, tail=...)``): the head streams a bf16 matrix, the embedding is a plain
-        bf16 table and no position encoding touches the embedding output."""
+        (``forward(step, tail=...)``): the parts say so themselves.  The embedding names a bf16
+        table that holds its outputs (``Embedding.pick_table``), no position encoding touches
+        the embedding output, and the head takes so many rows (``Head.can_pick``)."""
         spec = self.spec
-        table = getattr(spec.embedding, "table", None)
-        plain_embedding = (type(spec.embedding).__name__ == "TokenEmbedding" and table is not None
-                           and table.dtype == torch.bfloat16)
         untouched = all(type(p).on_embedding is Positions.on_embedding for p in spec.positions)
-        return (self.dtype == torch.bfloat16 and plain_embedding and untouched
-                and hasattr(spec.head, "can_pick") and spec.head.can_pick(rows))
+        return (self.dtype == torch.bfloat16 and untouched
+                and spec.embedding.pick_table() is not None and spec.head.can_pick(rows))
 
     def embed(self, step) -> torch.Tensor:
         """The step's residual stream, filled from the embedding."""

@@ -28,17 +28,10 @@ from kvforge_amd.registry import register_mixer
 KEYS_PER_CUT = 512
 MAX_CUTS = 64            # what the merge kernels take
 SKEW_MAX_CUTS = 8
-_compute_units: dict[int, int] = {}
 
 
 def compute_units(device) -> int:
-    """Compute units of the device the step runs on, asked of the device once."""
-    index = torch.device(device).index
-    if index is None:
-        index = torch.cuda.current_device()
-    if index not in _compute_units:
-        _compute_units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
-    return _compute_units[index]
+    return ops.compute_units(device)
 
 
 def skew_cuts(max_ctx: int, sum_ctx: int, n: int) -> int:

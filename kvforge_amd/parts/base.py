@@ -200,6 +200,43 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Turns token ids into the first residual stream.  ``hidden``: the stream's width."""
+
+    hidden: int
+
+    def forward(self, ids: torch.Tensor, out: torch.Tensor) -> None:
+        """``out[m]`` (fp32 ``[N, hidden]``) = the embedding of token ``ids[m]``."""
+        raise NotImplementedError
+
+    def pick_table(self) -> torch.Tensor | None:
+        """A bf16 table ``[vocab, hidden]`` whose row ``t``, widened to fp32, *is* what
+        ``forward`` gives for token ``t``, or ``None`` (the default) when no such table
+        exists.  A head whose kernel chooses the next token itself (``Head.pick``) gathers the
+        next step's residual rows from it; an embedding that says ``None`` keeps its model on
+        the path that samples from stored logits and embeds in a kernel of its own."""
+        return None
+
+
+class Head(Part):
+    """Turns normalised rows into logits over the vocabulary."""
+
+    def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
+        """``logits`` (fp32 ``[R, vocab]``) for the rows ``x [R, hidden]``."""
+        raise NotImplementedError
+
+    def can_pick(self, rows: int) -> bool:
+        """Whether ``pick`` takes ``rows`` rows (default: never)."""
+        return False
+
+    def pick(self, x: torch.Tensor, residual: torch.Tensor, step: "Step", tail) -> None:
+        """The tail of a greedy step of single tokens without stored logits: choose every row's
+        best token (the lowest index among equals), make it the sequence's next input in the
+        step's device buffers and leave its embedding (``tail.embed_table``) in ``residual``.
+        Only called where ``can_pick`` said yes."""
+        raise NotImplementedError
+
+
 class Block(Part):
     """An arrangement of parts around the residual stream."""
 
@@ -288,10 +325,10 @@ class ModelSpec:
     """Everything the registry's builder decides for one architecture."""
 
     config: object
-    embedding: Part
+    embedding: Embedding
     blocks: list[Block]
     final_norm: Norm
-    head: Part
+    head: Head
     positions: list[Positions] = field(default_factory=list)
     schedule: list[LayerCall] | None = None
     # checkpoint names that may be present and are not loaded (regular expressions)

@@ -5,10 +5,10 @@ from __future__ import annotations
 import torch
 
 from kvforge_amd.kernels import ops
-from kvforge_amd.parts.base import Part, WeightSpec
+from kvforge_amd.parts.base import Embedding, Head, WeightSpec
 
 
-class TokenEmbedding(Part):
+class TokenEmbedding(Embedding):
     """``h0 = table[ids]`` into the fp32 residual stream; no scaling."""
 
     replayable = True
@@ -32,8 +32,12 @@ class TokenEmbedding(Part):
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed(ids, self.table, out)
 
+    def pick_table(self) -> torch.Tensor | None:
+        t = self.table
+        return t if t is not None and t.dtype == torch.bfloat16 else None
 
-class LMHead(Part):
+
+class LMHead(Head):
     """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
     table when the head shares it (then no tensor of its own is expected)."""
 

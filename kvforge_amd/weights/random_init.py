@@ -16,12 +16,22 @@ import torch
 from kvforge_amd import registry
 from kvforge_amd.weights.io import write_safetensors
 
-_STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+_STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32,
+          torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
 
 
-def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.Tensor]:
-    """Tensors for every name the model expects, drawn in sorted name order from one generator."""
-    store = _STORE[dtype]
+def _stored_as(dtype: "str | torch.dtype") -> torch.dtype:
+    try:
+        return _STORE[dtype]
+    except KeyError:
+        raise ValueError(f"random weights are stored as bfloat16 or float32, not {dtype!r}") from None
+
+
+def random_tensors(spec, seed: int, dtype: "str | torch.dtype" = "bfloat16") -> dict[str, torch.Tensor]:
+    """Tensors for every name the model expects, drawn in 32-bit in sorted name order from one
+    generator and stored as ``dtype`` (the reference draws in 32-bit and casts to the engine's
+    type, src/tokenvault/model_loader.py:55-61)."""
+    store = _stored_as(dtype)
     gen = torch.Generator().manual_seed(int(seed))
     out: dict[str, torch.Tensor] = {}
     for name, w in sorted(spec.weight_specs().items()):
@@ -40,8 +50,10 @@ def random_tensors(spec, seed: int, dtype: str = "bfloat16") -> dict[str, torch.
 
 
 def write_random_model(folder: str, config: "dict[str, Any] | Any", seed: int = 0,
-                       dtype: str = "bfloat16") -> str:
-    """``config``: a config.json dictionary or a typed configuration."""
+                       dtype: "str | torch.dtype" = "bfloat16") -> str:
+    """``config``: a config.json dictionary or a typed configuration.  ``dtype``: what the
+    file stores; a float32 engine should be given ``"float32"``, or it only ever meets numbers
+    that bfloat16 can hold (``InferenceEngine.from_config`` passes its own type)."""
     cfg = registry.config_from_dict(config) if isinstance(config, dict) else config
     spec = registry.build_spec(cfg)
     cfg.save(folder)
@@ -50,15 +62,16 @@ def write_random_model(folder: str, config: "dict[str, Any] | Any", seed: int = 
 
 
 def load_random_weights(spec, seed: int, engine_dtype: torch.dtype, device: "torch.device | str",
-                        dtype: str = "bfloat16") -> None:
+                        dtype: "str | torch.dtype | None" = None) -> dict[str, torch.Tensor]:
     """The random-weights mode without the files, for models too large to be worth writing:
     every tensor of ``spec`` is drawn on ``device`` (same laws, same name order, stored in
-    ``dtype`` and then held as the loader would hold a tensor stored so) and handed to the
-    parts.  The device's generator gives other numbers than ``write_random_model`` does for the
-    same seed."""
+    ``dtype``, by default the engine's own, and then held as the loader would hold a tensor
+    stored so) and handed to the parts.  The device's generator gives other numbers than
+    ``write_random_model`` does for the same seed.  Returns the tensors by checkpoint name, as
+    drawn (the parts keep layouts of their own)."""
     from kvforge_amd.weights.loader import runtime_dtype
 
-    store = _STORE[dtype]
+    store = _stored_as(engine_dtype if dtype is None else dtype)
     gen = torch.Generator(device=device).manual_seed(int(seed))
     tensors: dict[str, torch.Tensor] = {}
     for name, w in sorted(spec.weight_specs().items()):
@@ -76,3 +89,4 @@ def load_random_weights(spec, seed: int, engine_dtype: torch.dtype, device: "tor
         tensors[name] = t.to(store).to(runtime_dtype(store, engine_dtype)).contiguous()
     for part in spec.all_parts():
         part.load(tensors)
+    return tensors

@@ -1,8 +1,10 @@
 """A plain, slow Llama decoder: whole sequences, no cache, one function per part, 32-bit torch
 on the CPU.  It is the oracle the engine is held to and shares no code with ``kvforge_amd``:
-it parses ``config.json`` itself and takes weights as a ``{checkpoint name: tensor}`` dict.
+it parses ``config.json`` itself and reads a folder's tensors with the ``safetensors`` package
+(``read_weights``), as a ``{checkpoint name: tensor}`` dict.
 
-Every function cites the lines of the reference (``/root/reference``) whose formula it follows.
+Every function cites the lines of the reference (``src/tokenvault/...``) whose formula it
+follows.
 The reference has no llama3 frequency scaling and no sliding window; those two follow the
 parameter names of the model's ``config.json`` and are pinned by invariants in the tests
 (``factor == 1`` is the identity, thresholds are continuous; a window as long as the sequence
@@ -30,6 +32,18 @@ def read_config(folder: str) -> dict[str, Any]:
     c.setdefault("rope_theta", 10000.0)
     c.setdefault("tie_word_embeddings", False)
     return c
+
+
+def read_weights(folder: str) -> dict[str, torch.Tensor]:
+    """Every tensor of every ``*.safetensors`` file in the folder, as stored, on the CPU."""
+    from safetensors.torch import load_file
+    out: dict[str, torch.Tensor] = {}
+    for name in sorted(os.listdir(folder)):
+        if name.endswith(".safetensors"):
+            out.update(load_file(os.path.join(folder, name)))
+    if not out:
+        raise FileNotFoundError(f"no .safetensors file in {folder}")
+    return out
 
 
 # --------------------------------------------------------------------------- parts

@@ -55,6 +55,34 @@ WIDE_C = dict(WIDE, vocab_size=500, hidden_size=256, num_hidden_layers=2, num_at
               num_key_value_heads=4, head_dim=128, intermediate_size=4096)
 
 
+_STORED: dict[tuple[str, str], str] = {}
+
+
+def stored_as(folder: str, dtype: str) -> str:
+    """The folder's model with its floating tensors stored as ``dtype`` ("float32" or
+    "bfloat16"): the folder itself if it stores them so, else a copy beside it, made once by
+    conversion.  A float32 engine is to be given weights that bfloat16 cannot hold, a bfloat16
+    engine weights stored in bfloat16 (one stored in 32-bit would stay 32-bit there)."""
+    import shutil
+    from safetensors.torch import save_file
+    want = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
+    key = (os.path.abspath(folder), dtype)
+    if key not in _STORED:
+        w = plain.read_weights(folder)
+        if all(t.dtype == want for t in w.values() if t.is_floating_point()):
+            _STORED[key] = folder
+        else:
+            twin = f"{folder.rstrip(os.sep)}.{dtype}"
+            os.makedirs(twin, exist_ok=True)
+            for name in os.listdir(folder):
+                if not name.endswith(".safetensors") and not name.endswith(".index.json"):
+                    shutil.copy(os.path.join(folder, name), os.path.join(twin, name))
+            save_file({k: (t.to(want) if t.is_floating_point() else t).contiguous() for k, t in w.items()},
+                      os.path.join(twin, "model.safetensors"), metadata={"format": "pt"})
+            _STORED[key] = twin
+    return _STORED[key]
+
+
 def sharpen(folder: str, factor: float) -> None:
     """Scale every q and k projection so that attention is peaked: with N(0, 0.02) weights the
     scores are nearly flat and one misplaced key would hide among hundreds."""
@@ -89,7 +117,7 @@ def liven(folder: str, qk: float = 6.0, out: float = 8.0) -> None:
 def context_matters(folder: str, prompts: list[list[int]], n: int = 6) -> bool:
     """Whether the plain model's greedy continuation of every prompt differs from the
     continuation of the prompt's last token alone."""
-    w = __import__("kvforge_amd").read_safetensors_folder(folder)
+    w = plain.read_weights(folder)
     cfg = plain.read_config(folder)
     return all(plain.greedy(w, cfg, p, n) != plain.greedy(w, cfg, p[-1:], n) for p in prompts if len(p) > 1)
 
@@ -213,7 +241,7 @@ def compare(folder: str, tb: TraceBuilder, out_dir: str, prompts: dict[str, list
     operations are rounded), and a row's absolute tolerance is no smaller than three times the
     largest difference that run shows from the 32-bit one in the same row.  A wrong key or page
     moves a row by about the logits' spread, many times that."""
-    w = {k: v for k, v in __import__("kvforge_amd").read_safetensors_folder(folder).items()}
+    w = {k: v for k, v in plain.read_weights(folder).items()}
     cfg = plain.read_config(folder)
     V = cfg["vocab_size"]
     by_tokens: dict[tuple, torch.Tensor] = {}

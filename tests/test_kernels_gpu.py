@@ -599,6 +599,32 @@ def test_gemm_generic_few_rows_over_long_and_uneven_k(m, tw):
     torch.testing.assert_close(acc.double(), want + 1.0, atol=3e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
+@pytest.mark.parametrize("n,k", [(6150, 516), (16390, 260)])
+@pytest.mark.parametrize("tw", DTYPES)
+def test_gemm_generic_few_rows_over_wide_weights(m, n, k, tw):
+    """The weight-streaming fp32 kernel changes its shape with the width of W: two columns per
+    wave from 6,144 columns on, four from 16,384 (the widths of gate/up and of the vocabulary).
+    32-bit weights that bfloat16 cannot hold, N that ends inside a wave's columns, against a
+    64-bit product; and the sums are the same whichever shape took them (a column of the wide
+    product equals the column computed over a narrow slice of W)."""
+    g = torch.Generator().manual_seed(n + m)
+    a = torch.randn(m, k, generator=g).to(DEV)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(tw).to(DEV)
+    if tw == torch.float32:
+        assert not torch.equal(w.bfloat16().float(), w)
+    want = a.double() @ w.double().T
+    out = torch.full((m, n), 7.0, device=DEV)
+    ops().gemm(a, w, out)
+    torch.testing.assert_close(out.double(), want, atol=2e-5, rtol=1e-5)
+    acc = torch.ones(m, n, device=DEV)
+    ops().gemm(a, w, acc, accumulate=True)
+    torch.testing.assert_close(acc.double(), want + 1.0, atol=2e-5, rtol=1e-5)
+    narrow = torch.empty(m, 100, device=DEV)
+    ops().gemm(a, w[n - 100:].contiguous(), narrow)
+    assert torch.equal(narrow, out[:, n - 100:])
+
+
 class Paged:
     """Scatters contiguous per-sequence K/V into shuffled pages: K ``[nb, KV, bs, d]``, V
     transposed ``[nb, KV, d, bs]``."""
@@ -735,11 +761,13 @@ def test_attn_decode(dtype, H, KV, d, bs, splits, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attn_decode_in_cuts_clears_the_rows_of_empty_sequences(dtype):
+@pytest.mark.parametrize("splits", [1, 4])
+def test_attn_decode_clears_the_rows_of_empty_sequences(dtype, splits):
     """A captured batch is padded with sequences that hold nothing.  With the key range in cuts
     their rows have no partial results; the merge must not read the workspace for them (it holds
-    whatever an earlier step left, NaNs here) and gives them zeros."""
-    H, KV, d, bs, splits = 8, 2, 64, 16, 4
+    whatever an earlier step left, NaNs here) and gives them zeros.  With the key range whole
+    their rows get zeros as well, not what an earlier step left in the output."""
+    H, KV, d, bs = 8, 2, 64, 16
     seq_lens = [70, 1, 600]
     paged = Paged(seq_lens, KV, d, bs, dtype, seed=3)
     table = torch.cat([paged.table, torch.full((2, paged.table.shape[1]), -1, dtype=torch.int32)])
@@ -754,7 +782,8 @@ def test_attn_decode_in_cuts_clears_the_rows_of_empty_sequences(dtype):
           torch.full((n * H * splits * 2,), float("nan"), device=DEV))
     out = torch.full((n, H * d), 7.0, dtype=dtype, device=DEV)
     ops().attn_decode(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), table.to(DEV), None, n, cu.to(DEV),
-                      ctx.to(DEV), out, H, KV, d, scale, 0, splits, ws, token_is_seq=True)
+                      ctx.to(DEV), out, H, KV, d, scale, 0, splits, ws if splits > 1 else None,
+                      token_is_seq=True)
     torch.testing.assert_close(out[:3].float().cpu(), want.reshape(3, H * d), **tol(dtype))
     assert bool((out[3:] == 0).all())
 

@@ -119,9 +119,9 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs, small_chip, m
     are scaled so the scores are peaked.  ``small_chip``: the part is told of a chip without any
     compute unit, which any rows fill, so it takes its items of two row tiles per wave
     where the kernel has them."""
-    from kvforge_amd.parts import attention
+    from kvforge_amd.kernels import ops as kernel_ops
     if small_chip:
-        monkeypatch.setattr(attention, "_compute_units", {i: 0 for i in range(torch.cuda.device_count())})
+        monkeypatch.setattr(kernel_ops, "_compute_units", {i: 0 for i in range(torch.cuda.device_count())})
     hidden = 40
     rot = RotaryPositions(d, 1000.0)
     rot.prepare(64, DEV)
@@ -325,7 +325,7 @@ def toy_folder(tmp_path_factory):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_toy_architecture_registers_builds_and_steps(toy_folder, dtype):
-    w = kvforge_amd.read_safetensors_folder(toy_folder)
+    w = plain.read_weights(toy_folder)
     model = Transformer.from_folder(toy_folder, dtype, DEV)
     assert isinstance(model.config, ToyConfig)
     # one cache group with one owner (call 0); calls 1 and 3 each hold a state of their own
@@ -359,7 +359,7 @@ def test_toy_architecture_registers_builds_and_steps(toy_folder, dtype):
 
 
 def test_toy_architecture_generates_through_the_engine(toy_folder):
-    w = kvforge_amd.read_safetensors_folder(toy_folder)
+    w = plain.read_weights(toy_folder)
     engine = kvforge_amd.InferenceEngine.from_folder(
         toy_folder, kvforge_amd.EngineConfig(
             cache=kvforge_amd.CacheConfig(block_size=4, num_blocks=64),

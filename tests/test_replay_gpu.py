@@ -36,12 +36,17 @@ def build_all_modes(prompts, seed):
 
 
 # with the weights as drawn (flat attention) the two given configurations are enough
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+# a float32 engine meets weights stored in 32-bit, which bfloat16 cannot hold; once it is given
+# weights stored in bfloat16 (widening at load is a path too)
+@pytest.mark.parametrize("dtype,store", [("float32", "float32"), ("bfloat16", "bfloat16"),
+                                         ("float32", "bfloat16")])
 @pytest.mark.parametrize("name,sharp", [(n, s) for n in CONFIGS for s in (0.0, 6.0) if s or n != "tiny-c"])
-def test_replay_all_modes(tmp_path, name, dtype, sharp):
+def test_replay_all_modes(tmp_path, name, dtype, store, sharp):
+    if store != dtype and (name, sharp) != ("tiny-b", 6.0):
+        pytest.skip("one configuration is enough for the widening load")
     make, seed, lengths = CONFIGS[name]
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, make(), seed=seed)
+    kvforge_amd.write_random_model(folder, make(), seed=seed, dtype=store)
     if sharp:
         ru.sharpen(folder, sharp)
     cfg = make()
@@ -75,7 +80,7 @@ def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, whic
         heads = cfg["num_attention_heads"] * cfg["head_dim"]
         assert ops.k_halves_pay(torch.empty(3, heads, dtype=bf), torch.empty(cfg["hidden_size"], heads, dtype=bf))
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, cfg, seed=4)
+    kvforge_amd.write_random_model(folder, cfg, seed=4, dtype=dtype)
     prompts = ru.random_prompts(cfg["vocab_size"], [41, 75, 52, 66], 9)
     tb, names = build_all_modes(prompts, 9)
     out = str(tmp_path / "out")
@@ -88,7 +93,7 @@ def test_replay_tiny_b_at_its_own_pages_of_eight_tokens(tmp_path, dtype):
     """Tiny B as its configuration has it: pages of 8 tokens (``--block-size 8``), all four ways
     of cutting the requests, with a pool so small that pages are used again."""
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1)
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1, dtype=dtype)
     ru.sharpen(folder, 6.0)
     prompts = ru.random_prompts(384, [1, 9, 40, 70, 129, 57], 1)
     tb, names = build_all_modes(prompts, 1)
@@ -107,7 +112,7 @@ def test_replay_an_id_that_ends_and_comes_back_with_other_tokens(tmp_path, dtype
     tables on the device, who the row belongs to; an id that returns must not be taken for its
     former self.  Every logit is compared with the plain model."""
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, dict(ru.TINY_C), seed=6)
+    kvforge_amd.write_random_model(folder, dict(ru.TINY_C), seed=6, dtype=dtype)
     ru.sharpen(folder, 6.0)
     p = ru.random_prompts(200, [90, 120, 70, 80], 21)
     first, y, z, other = p["p0"], p["p1"], p["p2"], p["p3"]
@@ -159,7 +164,7 @@ def test_replay_at_the_served_width(tmp_path, shape, dtype):
     large)."""
     cfg = SERVED[shape]()
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, cfg, seed=12)
+    kvforge_amd.write_random_model(folder, cfg, seed=12, dtype=dtype)
     # At these widths q.k already spreads over a few units (its spread grows with the width);
     # 1.5 makes the scores' spread about 2 (1B shape) and 4 (8B shape): peaked enough for one
     # wrong key to show, without multiplying the rounding of q and k into the logits.
@@ -198,7 +203,7 @@ def test_replay_first_tokens_and_one_token_requests(tmp_path):
     """The first tokens of a sequence: a request of one token, of two, a first step of one token
     followed by a portion, and position 0 decoded alone."""
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1)
+    kvforge_amd.write_random_model(folder, kvforge_amd.preset_dict("tiny-b"), seed=1, dtype="float32")
     ru.sharpen(folder, 6.0)
     prompts = ru.random_prompts(384, [1, 2, 20, 17], 5)
     tb = ru.TraceBuilder()
@@ -210,8 +215,9 @@ def test_replay_first_tokens_and_one_token_requests(tmp_path):
             end=["p2", "p3"])
     for dtype in ("float32", "bfloat16"):
         out = str(tmp_path / dtype)
-        ru.run_trace(folder, dtype, tb, out)
-        ru.compare(folder, tb, out, prompts, *TOL[dtype])
+        stored = ru.stored_as(folder, dtype)
+        ru.run_trace(stored, dtype, tb, out)
+        ru.compare(stored, tb, out, prompts, *TOL[dtype])
 
 
 def test_replay_decoding_with_split_key_range(tmp_path):
@@ -219,7 +225,7 @@ def test_replay_decoding_with_split_key_range(tmp_path):
     kernel cut the key range into several runs that are merged afterwards."""
     cfg = dict(ru.TINY_C, max_position_embeddings=2048)
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, cfg, seed=5)
+    kvforge_amd.write_random_model(folder, cfg, seed=5, dtype="float32")
     ru.sharpen(folder, 6.0)
     prompts = ru.random_prompts(200, [1240], 11)
     tb = ru.TraceBuilder()
@@ -229,15 +235,16 @@ def test_replay_decoding_with_split_key_range(tmp_path):
         tb.step([("p0", [prompts["p0"][1200 + i]], [0])], end=["p0"] if i == 39 else [])
     for dtype in ("float32", "bfloat16"):
         out = str(tmp_path / dtype)
-        ru.run_trace(folder, dtype, tb, out)
-        ru.compare(folder, tb, out, prompts, *TOL[dtype])
+        stored = ru.stored_as(folder, dtype)
+        ru.run_trace(stored, dtype, tb, out)
+        ru.compare(stored, tb, out, prompts, *TOL[dtype])
 
 
 def test_replay_long_decoding(tmp_path):
     """Two requests decoded token by token for 300 steps past a short prompt, across many
     pages."""
     folder = str(tmp_path / "model")
-    kvforge_amd.write_random_model(folder, ru.TINY_C, seed=3)
+    kvforge_amd.write_random_model(folder, ru.TINY_C, seed=3, dtype="float32")
     ru.sharpen(folder, 6.0)
     prompts = ru.random_prompts(200, [330, 318], 7)
     tb = ru.TraceBuilder()
@@ -247,5 +254,6 @@ def test_replay_long_decoding(tmp_path):
                 end=["p0", "p1"] if i == 299 else [])
     for dtype in ("float32", "bfloat16"):
         out = str(tmp_path / dtype)
-        ru.run_trace(folder, dtype, tb, out)
-        ru.compare(folder, tb, out, prompts, *TOL[dtype])
+        stored = ru.stored_as(folder, dtype)
+        ru.run_trace(stored, dtype, tb, out)
+        ru.compare(stored, tb, out, prompts, *TOL[dtype])

@@ -127,6 +127,50 @@ def test_without_chunking_a_prompt_waits_for_a_step_it_fits_in():
     assert shares(d.plan()) == [("b", 10)]
 
 
+def test_without_chunking_a_preempted_request_that_outgrew_the_budget_is_fed_in_portions():
+    """The reference refuses at the door what exceeds the budget by its prompt alone
+    (src/tokenvault/scheduler.py:109-129) but looks at prompt plus outputs when a preempted
+    request comes back (:206-207): a request that was preempted after it had grown past the
+    budget would then stand at the head of the line for ever.  Here it is fed again in portions.
+    5 pages of 4 tokens, 8 tokens a step, two prompts of 7 tokens with 12 new tokens each."""
+    d = Driver(num_blocks=5, block_size=4, max_num_batched_tokens=8, enable_chunked_prefill=False)
+    a = d.add("a", 7, 0.0, max_tokens=12)
+    b = d.add("b", 7, 1.0, max_tokens=12)
+    preempted_at, fed_again = None, []
+    for step in range(80):
+        if not d.sched.has_unfinished():
+            break
+        plan = d.step()
+        assert not plan.is_empty or plan.preempted, f"nothing planned at step {step}"
+        assert plan.num_tokens <= 8
+        if plan.preempted:
+            assert [r.request_id for r in plan.preempted] == ["b"]
+            preempted_at = (step, b.num_tokens)
+        elif preempted_at and len(fed_again) < 2:
+            fed_again += [(s.start, s.count, s.samples) for s in plan.slices if s.request is b]
+    assert preempted_at is not None and preempted_at[1] > 8          # it had outgrown a step
+    assert fed_again == [(0, 8, False), (8, preempted_at[1] - 8, True)]
+    assert a.finish_reason is FinishReason.LENGTH and b.finish_reason is FinishReason.LENGTH
+    assert a.num_output_tokens == b.num_output_tokens == 12
+    assert d.cache.num_free_blocks == 5
+
+
+def test_without_chunking_a_preempted_request_that_still_fits_a_step_comes_back_whole():
+    d = Driver(num_blocks=5, block_size=4, max_num_batched_tokens=16, enable_chunked_prefill=False)
+    d.add("a", 7, 0.0, max_tokens=12)
+    b = d.add("b", 7, 1.0, max_tokens=12)
+    whole = None
+    for _ in range(80):
+        if not d.sched.has_unfinished():
+            break
+        plan = d.step()
+        for s in plan.slices:
+            if s.request is b and b.num_preemptions and not s.decode and whole is None:
+                whole = (s.start, s.count, s.samples)
+    assert b.num_preemptions == 1 and whole == (0, whole[1], True) and whole[1] > 7
+    assert d.cache.num_free_blocks == 5
+
+
 def test_a_step_without_admission_leaves_arrivals_in_line():
     """``schedule(admit=False)`` and ``schedule(queued_steps=n)``: only what runs is planned."""
     d = Driver()

@@ -139,7 +139,7 @@ def latent_folder(tmp_path_factory):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_a_mixer_with_pages_of_its_own_make(latent_folder, dtype):
-    w = kvforge_amd.read_safetensors_folder(latent_folder)
+    w = plain.read_weights(latent_folder)
     model = Transformer.from_folder(latent_folder, dtype, DEV)
     # two groups: the two latent layers share one make of page, attention has another
     made = {tuple(t.name for t in g.pages): g.layers for g in model.cache_groups}
@@ -181,7 +181,7 @@ def test_a_mixer_with_pages_of_its_own_make(latent_folder, dtype):
 
 
 def test_the_latent_model_generates_through_the_engine(latent_folder):
-    w = kvforge_amd.read_safetensors_folder(latent_folder)
+    w = plain.read_weights(latent_folder)
     engine = kvforge_amd.InferenceEngine.from_folder(
         latent_folder, kvforge_amd.EngineConfig(
             dtype="float32", cache=kvforge_amd.CacheConfig(block_size=4, num_blocks=48),

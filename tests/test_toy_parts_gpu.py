@@ -257,7 +257,7 @@ def mix_folder(tmp_path_factory):
 def test_routing_spreads_over_experts(mix_folder):
     """The random router must not send everything to one pair, or the comparison below would
     not see a wrong choice."""
-    w = {k: v.float() for k, v in kvforge_amd.read_safetensors_folder(mix_folder).items()}
+    w = {k: v.float() for k, v in plain.read_weights(mix_folder).items()}
     x = torch.randn(64, 40, generator=torch.Generator().manual_seed(0))
     first = (x @ w["l.0.ff.router.weight"].T).argmax(-1)
     assert len(set(first.tolist())) == 3
@@ -265,7 +265,7 @@ def test_routing_spreads_over_experts(mix_folder):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_toy_parts_step_in_portions(mix_folder, dtype):
-    w = kvforge_amd.read_safetensors_folder(mix_folder)
+    w = plain.read_weights(mix_folder)
     model = Transformer.from_folder(mix_folder, dtype, DEV)
     kinds = [type(b).__name__ for b in model.spec.blocks]
     assert kinds == ["PreNormBlock", "ToyParallelBlock", "PreNormBlock"]
@@ -302,7 +302,7 @@ def test_toy_parts_step_in_portions(mix_folder, dtype):
 def test_toy_parts_generate_through_the_engine(mix_folder):
     """Greedy generation, decode steps replayed from graphs in runs: every produced token is the
     plain model's best (within rounding) at its place."""
-    w = kvforge_amd.read_safetensors_folder(mix_folder)
+    w = plain.read_weights(mix_folder)
     engine = kvforge_amd.InferenceEngine.from_folder(
         mix_folder, kvforge_amd.EngineConfig(
             dtype="float32", cache=kvforge_amd.CacheConfig(block_size=4, num_blocks=64),

@@ -126,7 +126,7 @@ def slopes_folder(tmp_path_factory):
 
 
 def test_the_bias_decides_the_logits(slopes_folder):
-    w = kvforge_amd.read_safetensors_folder(slopes_folder)
+    w = plain.read_weights(slopes_folder)
     ids = torch.randint(0, 83, (60,), generator=torch.Generator().manual_seed(1)).tolist()
     a, b = slopes_plain(w, ids), slopes_plain(w, ids, with_bias=False)
     assert float((a - b).abs().max()) > 0.3               # five times the widest tolerance below
@@ -135,7 +135,7 @@ def test_the_bias_decides_the_logits(slopes_folder):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_slopes_model_in_portions_with_pages_used_again(slopes_folder, dtype):
-    w = kvforge_amd.read_safetensors_folder(slopes_folder)
+    w = plain.read_weights(slopes_folder)
     model = Transformer.from_folder(slopes_folder, dtype, DEV)
     assert len(model.cache_groups) == 2                  # whole-context layers and window layers
     bs = 8
@@ -171,7 +171,7 @@ def test_slopes_model_in_portions_with_pages_used_again(slopes_folder, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_slopes_model_generates_through_captured_steps(slopes_folder, dtype):
-    w = kvforge_amd.read_safetensors_folder(slopes_folder)
+    w = plain.read_weights(slopes_folder)
     engine = kvforge_amd.InferenceEngine.from_folder(
         slopes_folder, kvforge_amd.EngineConfig(
             dtype=dtype, cache=kvforge_amd.CacheConfig(block_size=8, num_blocks=64),
