@@ -151,16 +151,25 @@ def swiglu(x: torch.Tensor, gate_w: torch.Tensor, up_w: torch.Tensor,
 def attention_block(x: torch.Tensor, w: dict[str, torch.Tensor], prefix: str, cfg: dict,
                     cos: torch.Tensor, sin: torch.Tensor, window: int | None,
                     store: torch.dtype | None = None,
-                    out_store: torch.dtype | None = None) -> torch.Tensor:
+                    out_store: torch.dtype | None = None,
+                    query_block: int | None = None) -> torch.Tensor:
     """src/tokenvault/model.py:77-92 without the cache: project, rotate q and k, attend,
-    project out."""
+    project out.  ``query_block``: attend that many queries at a time (each over the keys up to
+    its block's end), so that the scores of a sequence of tens of thousands of tokens never
+    exist all at once; the same numbers."""
     T = x.shape[0]
     H, KV, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     q = _stored(x @ w[prefix + "q_proj.weight"].to(x.dtype).T, store).view(T, H, d)
     k = _stored(x @ w[prefix + "k_proj.weight"].to(x.dtype).T, store).view(T, KV, d)
     v = _stored(x @ w[prefix + "v_proj.weight"].to(x.dtype).T, store).view(T, KV, d)
     q, k = _stored(apply_rope(q, cos, sin), store), _stored(apply_rope(k, cos, sin), store)
-    out = _stored(causal_attention(q, k, v, 1.0 / math.sqrt(d), 0, window), store)
+    if query_block is None:
+        out = causal_attention(q, k, v, 1.0 / math.sqrt(d), 0, window)
+    else:
+        out = torch.cat([causal_attention(q[lo:lo + query_block], k[:lo + query_block], v[:lo + query_block],
+                                          1.0 / math.sqrt(d), lo, window)
+                         for lo in range(0, T, query_block)])
+    out = _stored(out, store)
     return _stored(out.reshape(T, H * d) @ w[prefix + "o_proj.weight"].to(x.dtype).T, out_store)
 
 
@@ -182,8 +191,10 @@ def layer_window(cfg: dict, i: int) -> int | None:
 
 def forward(w: dict[str, torch.Tensor], cfg: dict, token_ids: list[int],
             first_position: int = 0, dtype: torch.dtype = torch.float32,
-            residual_in_fp32: bool = False) -> torch.Tensor:
-    """src/tokenvault/model.py:175-191 for one whole sequence: logits ``[T, vocab]`` in fp32.
+            residual_in_fp32: bool = False, query_block: int | None = None,
+            last: int | None = None) -> torch.Tensor:
+    """src/tokenvault/model.py:175-191 for one whole sequence: logits ``[T, vocab]`` in fp32
+    (of the last ``last`` positions only, if given; ``query_block``: see ``attention_block``).
     ``first_position`` shifts every position (only distances count under rotary).
     ``dtype=torch.float64`` computes everything but the rotary angles (which are 32-bit by
     definition) in double precision.  ``dtype=torch.bfloat16`` gives what the reference computes
@@ -206,10 +217,12 @@ def forward(w: dict[str, torch.Tensor], cfg: dict, token_ids: list[int],
         p = f"model.layers.{i}."
         a = _stored(rms_norm(h, w[p + "input_layernorm.weight"], eps), store)
         h = _stored(h + attention_block(a, w, p + "self_attn.", cfg, cos, sin,
-                                        layer_window(cfg, i), store, stream), stream)
+                                        layer_window(cfg, i), store, stream, query_block), stream)
         m = _stored(rms_norm(h, w[p + "post_attention_layernorm.weight"], eps), store)
         h = _stored(h + swiglu(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                                w[p + "mlp.down_proj.weight"], store, stream), stream)   # model.py:186-187
+    if last is not None:
+        h = h[-last:]
     hidden = _stored(rms_norm(h, w["model.norm.weight"], eps), store)    # model.py:188
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return _stored(hidden @ head.to(hidden.dtype).T, stream)            # model.py:157-158,190-191

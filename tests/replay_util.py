@@ -222,7 +222,7 @@ def run_trace(folder: str, dtype: str, tb: TraceBuilder, out_dir: str, max_token
 
 
 def compare(folder: str, tb: TraceBuilder, out_dir: str, prompts: dict[str, list[int]], atol: float,
-            rtol: float, measured_rounding: "bool | str" = False) -> float:
+            rtol: float, measured_rounding: "bool | str" = False, query_block: int | None = None) -> float:
     """Every row trace_run wrote against the plain model's logits at that request's position.
     Reports the first wrong place by step, request and position.
 
@@ -240,7 +240,10 @@ def compare(folder: str, tb: TraceBuilder, out_dir: str, prompts: dict[str, list
     (``plain.forward(dtype=bfloat16, residual_in_fp32=True)``: only the tensors between
     operations are rounded), and a row's absolute tolerance is no smaller than three times the
     largest difference that run shows from the 32-bit one in the same row.  A wrong key or page
-    moves a row by about the logits' spread, many times that."""
+    moves a row by about the logits' spread, many times that.
+
+    ``query_block``: the plain model attends so many queries at a time (for sequences whose
+    scores would not fit in memory all at once)."""
     w = {k: v for k, v in plain.read_weights(folder).items()}
     cfg = plain.read_config(folder)
     V = cfg["vocab_size"]
@@ -249,13 +252,14 @@ def compare(folder: str, tb: TraceBuilder, out_dir: str, prompts: dict[str, list
     for rid, toks in prompts.items():
         key = tuple(toks)
         if key not in by_tokens:
-            ref = plain.forward(w, cfg, toks)
+            ref = plain.forward(w, cfg, toks, query_block=query_block)
             floor = 0.0
             if measured_rounding == "bfloat16":
-                least = plain.forward(w, cfg, toks, dtype=torch.bfloat16, residual_in_fp32=True)
+                least = plain.forward(w, cfg, toks, dtype=torch.bfloat16, residual_in_fp32=True,
+                                      query_block=query_block)
                 floor = 3.0 * (least - ref).abs().max(dim=1).values          # per row
             elif measured_rounding:
-                exact = plain.forward(w, cfg, toks, dtype=torch.float64)
+                exact = plain.forward(w, cfg, toks, dtype=torch.float64, query_block=query_block)
                 floor = 5.0 * float((ref.double() - exact).abs().max())
                 ref = exact.float()
             by_tokens[key] = (ref, floor)

@@ -270,3 +270,19 @@ def test_draw_and_uniform():
     assert all(0 <= u < 1 for u in us) and abs(sum(us) / 2000 - 0.5) < 0.03
     assert plain_sampling.uniform(1, 2, 3) == plain_sampling.uniform(1, 2, 3)
     assert plain_sampling.uniform(1, 2, 3) != plain_sampling.uniform(1, 3, 3)
+
+
+def test_attention_in_query_blocks_gives_the_same_logits():
+    """``forward(query_block=...)`` never holds all scores at once (for sequences of tens of
+    thousands of tokens); it is the same computation, also with a window and with ``last``."""
+    cfg = dict(CFG, layer_types=["sliding_attention", "full_attention"], sliding_window=5)
+    w = tiny_weights(CFG)
+    ids = [(7 * i + 3) % 50 for i in range(37)]
+    for c in (CFG, cfg):
+        # in float64, where two orders of summation differ by nothing that could hide a mistake
+        f64 = dict(dtype=torch.float64)
+        full = plain.forward(w, c, ids, **f64)
+        for block in (1, 8, 37, 64):
+            torch.testing.assert_close(plain.forward(w, c, ids, query_block=block, **f64), full, atol=1e-7, rtol=1e-7)
+        torch.testing.assert_close(plain.forward(w, c, ids, query_block=8, last=5, **f64), full[-5:],
+                                   atol=1e-7, rtol=1e-7)

@@ -257,3 +257,46 @@ def test_replay_long_decoding(tmp_path):
         stored = ru.stored_as(folder, dtype)
         ru.run_trace(stored, dtype, tb, out)
         ru.compare(stored, tb, out, prompts, *TOL[dtype])
+
+
+LONG = {  # small layers around attention heads of the size long contexts are served with
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": 200,
+    "hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 2, "num_key_value_heads": 1,
+    "head_dim": 128, "intermediate_size": 96, "max_position_embeddings": 40960,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+    "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": False,
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_a_prompt_of_32k_tokens_in_portions_then_token_by_token(tmp_path, dtype):
+    """A prompt of 32,768 tokens is fed in sixteen portions of 2,048 and then goes on for 16
+    tokens one by one, a short request beside it for the second half (so the single-token steps
+    hold a context of 32k beside one of a few dozen): page numbers past 2,000 per request, query
+    runs at the end of tens of thousands of keys, the key range of one token in many cuts.
+    Attention is peaked (q and k scaled), so that keys far back carry weight.  All logits of
+    the last portion and of the single tokens, and some of every other portion, against the
+    plain model computed a block of queries at a time; the tolerance is measured as for the
+    served widths, since a softmax over 32k terms rounds differently in any two orders."""
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, dict(LONG), seed=15, dtype=dtype)
+    ru.sharpen(folder, 6.0)
+    prompts = ru.random_prompts(200, [32768 + 16, 56], 17)
+    big, small = prompts["p0"], prompts["p1"]
+    tb = ru.TraceBuilder()
+    for i in range(16):
+        lo = i * 2048
+        want = list(range(2048)) if i == 15 else [0, 1000, 2047]
+        entries = [("p0", big[lo:lo + 2048], want)]
+        if i == 8:
+            entries.append(("p1", small[:40], [0, 39]))
+        tb.step(entries)
+    for i in range(16):
+        tb.step([("p1", [small[40 + i]], [0]), ("p0", [big[32768 + i]], [0])],
+                end=["p0", "p1"] if i == 15 else [])
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, dtype, tb, out)
+    ru.compare(folder, tb, out, prompts, *TOL[dtype], measured_rounding=True if dtype == "float32" else dtype,
+               query_block=512)
