@@ -1,101 +1,131 @@
-// Paged causal attention for query runs of any length, computed on the vector ALUs in fp32.
-// It is the attention of the true 32-bit path and takes bf16 operands as well.
+// Paged attention of the true 32-bit path: every product and sum in fp32.  It takes bf16
+// operands as well (widened exactly), for caches whose pages the bf16 kernels do not take.
 //
-// One workgroup handles 16 "rows" of one (sequence, kv head): row r of a sequence is
-// (query token r / G, head r % G of the kv head's group), so the G query heads that share a
-// kv head also share every K/V tile the workgroup loads.  Keys are walked in tiles aligned
-// to multiples of the tile size from position 0, with a running maximum, sum and accumulator
-// per row (all fp32).  Key j is visible to the query at position p iff j <= p, j < context
-// length and, with a window w > 0, j > p - w.  Scores are scaled after the dot product; with
-// `slopes` (one number per q head) slopes[h] * (j - p) is added to them, a bias by distance.
+// Query runs of any length (attn_mfma32_kernel): fp32 on the matrix cores with
+// v_mfma_f32_16x16x4_f32, which multiplies and adds in fp32.  Row r of a sequence is
+// (query token r / G, head r % G of the kv head's group), so the G query heads that share a kv
+// head also share every K/V tile.  A workgroup of four waves takes an item of 64 rows of one
+// (sequence, kv head), a wave 16 of them.  Keys are walked in tiles aligned to multiples of the
+// tile size from position 0; the tile's keys, then its values, are staged in LDS for the four
+// waves.  A wave computes the transposed scores S^T = K Q^T (keys down the instruction's rows),
+// so that a lane ends up with four neighbouring keys of one query row: the running maximum and
+// sum of a row are a lane's own, the probabilities stay in registers and are the right-hand
+// operand of O^T += V^T P as they are.  Key j is visible to the query at position p iff j <= p,
+// j < context length and, with a window w > 0, j > p - w.  Scores are scaled after the dot
+// product; with `slopes` (one number per q head) slopes[h] * (j - p) is added to them, a bias by
+// distance.  The order of every sum is fixed by the positions alone.
 //
 // K pages are [num_blocks, KV, block_size, d], V pages are transposed [num_blocks, KV, d,
-// block_size]; a key whose page entry is negative or out of range contributes nothing.
+// block_size]; a key whose page entry is negative or out of range reads as zeros.
 #include "common.h"
 
 namespace {
-constexpr int ROWS = 16;
+constexpr int ITEM_ROWS = 64;   // rows per work item: four waves of 16
 
 struct AttnArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs;
-  int tiles_per_seq;  // 0: `work` holds (sequence, tile, tile or -1) rows; > 0: `work` lists sequences (or
-                      // is null for 0, 1, 2, ...) and each takes this many tiles
   float scale;
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
 };
 
-template <typename T, int DMAX, int BKEYS>
-__global__ __launch_bounds__(256) void attn_tile_kernel(
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// four consecutive elements as floats; p on 16 bytes (fp32) / 8 bytes (bf16)
+__device__ __forceinline__ f32x4 load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 load4(const bf16_t* p) {
+  const uint2 r = *reinterpret_cast<const uint2*>(p);
+  return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+               __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, f32x4 v) {
+  uint2 r;
+  r.x = static_cast<uint32_t>(f32_to_bf16(v[0])) | (static_cast<uint32_t>(f32_to_bf16(v[1])) << 16);
+  r.y = static_cast<uint32_t>(f32_to_bf16(v[2])) | (static_cast<uint32_t>(f32_to_bf16(v[3])) << 16);
+  *reinterpret_cast<uint2*>(p) = r;
+}
+
+// The instruction: D[i][j] += sum_k A[i][k] B[k][j] over k = 0..3; lane l gives A[l % 16][l / 16]
+// and B[l / 16][l % 16] and holds D[4 (l / 16) + v][l % 16], v = 0..3.  Here the four lane
+// groups stand for four *neighbouring* k each (group g takes k = 4 g + e in instruction e of
+// four), so that a lane's operands are 16 consecutive bytes.
+__device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+template <typename T, int DMAX>
+__global__ __launch_bounds__(256) void attn_mfma32_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, const int* __restrict__ cu_q,
     const int* __restrict__ ctx_lens, const int* __restrict__ work, T* __restrict__ out,
     AttnArgs a) {
-  __shared__ float Qs[ROWS][DMAX + 1];
-  __shared__ float KVs[BKEYS][DMAX + 1];
-  __shared__ float Ps[ROWS][BKEYS + 1];
+  constexpr int DT = DMAX / 16;                // 16-element tiles of the head
+  constexpr int BK = DMAX > 128 ? 32 : 64;     // keys per tile
+  constexpr int ST = BK / 16;                  // 16-key blocks per tile
+  constexpr int KLD = DMAX + 4, VLD = BK + 4;  // LDS rows 16 bytes apart in the banks
+  constexpr int FLOATS = BK * KLD > DMAX * VLD ? BK * KLD : DMAX * VLD;
+  __shared__ __align__(16) float KVs[FLOATS];  // the tile's keys [BK][KLD], then its values [d][VLD]
 
-  int seq, tile;
-  if (a.tiles_per_seq > 0) {
-    const int idx = blockIdx.x / a.tiles_per_seq;
-    seq = work ? work[idx] : idx;
-    tile = blockIdx.x - idx * a.tiles_per_seq;
-  } else {
-    // rows (sequence, tile, tile or -1): two workgroups per row, one for each tile
-    const int w = blockIdx.x >> 1;
-    seq = work[3 * w];
-    tile = work[3 * w + 1 + (blockIdx.x & 1)];
-    if (tile < 0) return;
-  }
-  if (seq < 0 || seq >= a.n_seqs) return;
+  // rows (sequence, item, item or -1): two workgroups per row, one for each item
+  const int w = blockIdx.x >> 1;
+  const int seq = work[3 * w];
+  const int item = work[3 * w + 1 + (blockIdx.x & 1)];
+  if (item < 0 || seq < 0 || seq >= a.n_seqs) return;
   const int kvh = blockIdx.y;
   const int G = a.H / a.KV, D = a.d;
   const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
   const int start = ctx - qlen;  // position of the run's first query
-  const int rows_total = qlen * G, r0 = tile * ROWS;
-  if (r0 >= rows_total || qlen <= 0 || start < 0) return;
+  const int rows_total = qlen * G, item0 = item * ITEM_ROWS;
+  if (item0 >= rows_total || qlen <= 0 || start < 0) return;
 
-  const int tid = threadIdx.x;
-  const int r = tid / 16, c16 = tid % 16;
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / KVF_WAVE);
+  const int j16 = lane % 16, g4 = lane / 16;
   const int* table = block_table + static_cast<size_t>(seq) * a.table_stride;
 
-  // stage the query rows
-  for (int idx = tid; idx < ROWS * D; idx += 256) {
-    const int rr = idx / D, kk = idx - rr * D;
-    const int row = r0 + rr;
-    float v = 0.f;
-    if (row < rows_total) {
-      const int i = row / G, g = row - i * G;
-      v = Elem<T>::load(q + static_cast<size_t>(q0 + i) * a.q_stride + (kvh * G + g) * D + kk);
-    }
-    Qs[rr][kk] = v;
+  // this lane's query row (the same in the four lane groups)
+  const int r0 = item0 + wave * 16;
+  const int row = r0 + j16;
+  const bool row_ok = row < rows_total;
+  const int tok = row_ok ? row / G : 0;
+  const int head = kvh * G + (row_ok ? row - tok * G : 0);
+  const int pos = start + tok;
+  const float slope = a.slopes && row_ok ? a.slopes[head] : 0.f;
+  // key ranges: of the workgroup's rows (what is staged) and of this wave's (what it works on)
+  int last = item0 + ITEM_ROWS - 1;
+  if (last >= rows_total) last = rows_total - 1;
+  const int hi = min(start + last / G, ctx - 1);
+  int lo = 0;
+  if (a.window > 0) lo = max(0, start + item0 / G - a.window + 1);
+  int hi_w = -1, lo_w = 0;
+  if (r0 < rows_total) {
+    int last_w = r0 + 15;
+    if (last_w >= rows_total) last_w = rows_total - 1;
+    hi_w = min(start + last_w / G, ctx - 1);
+    if (a.window > 0) lo_w = max(0, start + r0 / G - a.window + 1);
   }
 
-  const int my_row = r0 + r;
-  const bool row_ok = my_row < rows_total;
-  const int my_pos = start + (row_ok ? my_row / G : 0);
-  const float slope = a.slopes && row_ok ? a.slopes[kvh * G + my_row % G] : 0.f;
-  const int pos_min = start + r0 / G;
-  int last_row = r0 + ROWS - 1;
-  if (last_row >= rows_total) last_row = rows_total - 1;
-  const int pos_max = start + last_row / G;
-  int lo = 0;
-  if (a.window > 0) {
-    lo = pos_min - a.window + 1;
-    if (lo < 0) lo = 0;
+  // the query row's elements 16 u + 4 g4 .. + 3, u = 0 .. DT - 1
+  f32x4 qf[DT];
+  {
+    const T* qp = q + static_cast<size_t>(q0 + tok) * a.q_stride + head * D + 4 * g4;
+#pragma unroll
+    for (int u = 0; u < DT; ++u)
+      qf[u] = (row_ok && 16 * u < D) ? load4(qp + 16 * u) : f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  const int hi = pos_max < ctx - 1 ? pos_max : ctx - 1;  // last key any row may see
 
   float m_run = -INFINITY, l_run = 0.f;
-  float acc[DMAX / 16];
+  f32x4 acc[DT];   // acc[t][v]: element 16 t + 4 g4 + v of this lane's row
 #pragma unroll
-  for (int j = 0; j < DMAX / 16; ++j) acc[j] = 0.f;
+  for (int t = 0; t < DT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int chunks_per_key = D / 8;
-  for (int t0 = (lo / BKEYS) * BKEYS; t0 <= hi; t0 += BKEYS) {
-    // ---- K tile
-    __syncthreads();
-    for (int ch = tid; ch < BKEYS * chunks_per_key; ch += 256) {
-      const int c = ch / chunks_per_key, k8 = (ch - c * chunks_per_key) * 8;
+  const bool quads = a.block_size % 4 == 0;
+  const int chunks = D / 8;
+  for (int t0 = (lo / BK) * BK; t0 <= hi; t0 += BK) {
+    // ---- keys of the tile
+    __syncthreads();   // the values of the tile before have been used
+    for (int ch = tid; ch < BK * chunks; ch += 256) {
+      const int c = ch / chunks, k8 = (ch - c * chunks) * 8;
       const int j = t0 + c;
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (j >= lo && j <= hi) {
@@ -105,81 +135,117 @@ __global__ __launch_bounds__(256) void attn_tile_kernel(
           load8(k_pages + ((static_cast<size_t>(page) * a.KV + kvh) * a.block_size +
                            (j - blk * a.block_size)) * D + k8, v);
       }
-#pragma unroll
-      for (int e = 0; e < 8; ++e) KVs[c][k8 + e] = v[e];
+      *reinterpret_cast<float4*>(&KVs[c * KLD + k8]) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(&KVs[c * KLD + k8 + 4]) = make_float4(v[4], v[5], v[6], v[7]);
     }
     __syncthreads();
-    // ---- scores for row r, keys c16 + 16*jj
-    float s[BKEYS / 16];
+    const bool mine = t0 <= hi_w && t0 + BK > lo_w;   // the same in all lanes of the wave
+    f32x4 p[ST];
+    float corr = 1.f;
+    if (mine) {
+      // ---- transposed scores: p[st][v] = key t0 + 16 st + 4 g4 + v against this lane's row
+      float tmax = -INFINITY;
 #pragma unroll
-    for (int jj = 0; jj < BKEYS / 16; ++jj) s[jj] = 0.f;
-    for (int kk = 0; kk < D; ++kk) {
-      const float qv = Qs[r][kk];
+      for (int st = 0; st < ST; ++st) {
+        f32x4 sc = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int jj = 0; jj < BKEYS / 16; ++jj) s[jj] = fmaf(qv, KVs[c16 + 16 * jj][kk], s[jj]);
+        for (int u = 0; u < DT; ++u) {
+          if (16 * u >= D) break;
+          const f32x4 kf = *reinterpret_cast<const f32x4*>(&KVs[(16 * st + j16) * KLD + 16 * u + 4 * g4]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sc = mfma4(kf[e], qf[u][e], sc);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int j = t0 + 16 * st + 4 * g4 + v;
+          bool vis = row_ok && j <= pos && j < ctx;
+          if (a.window > 0) vis = vis && (j > pos - a.window);
+          sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), sc[v] * a.scale) : -INFINITY;
+          tmax = fmaxf(tmax, sc[v]);
+        }
+        p[st] = sc;
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, KVF_WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, KVF_WAVE));
+      const float m_new = fmaxf(m_run, tmax);
+      float psum = 0.f;
+      if (m_new == -INFINITY) {
+#pragma unroll
+        for (int st = 0; st < ST; ++st) p[st] = f32x4{0.f, 0.f, 0.f, 0.f};
+      } else {
+        corr = expf(m_run - m_new);  // exp(-inf) = 0 on the first visible tile
+#pragma unroll
+        for (int st = 0; st < ST; ++st)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float e = expf(p[st][v] - m_new);
+            p[st][v] = e;
+            psum += e;
+          }
+      }
+      psum += __shfl_xor(psum, 16, KVF_WAVE);
+      psum += __shfl_xor(psum, 32, KVF_WAVE);
+      l_run = l_run * corr + psum;
+      m_run = m_new;
     }
-    float tmax = -INFINITY;
+    // ---- values of the tile (over the keys, once every wave has finished with them)
+    __syncthreads();
+    if (quads) {
+      // four neighbouring keys of one element lie side by side in a page
+      for (int idx = tid; idx < D * (BK / 4); idx += 256) {
+        const int e = idx / (BK / 4), c = (idx - e * (BK / 4)) * 4;
+        const int j = t0 + c;
+        f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (j + 3 >= lo && j <= hi) {
+          const int blk = j / a.block_size;
+          const int page = blk < a.table_stride ? table[blk] : -1;
+          if (page >= 0 && page < a.num_blocks) {
+            v = load4(v_pages + ((static_cast<size_t>(page) * a.KV + kvh) * D + e) * a.block_size +
+                      (j - blk * a.block_size));
 #pragma unroll
-    for (int jj = 0; jj < BKEYS / 16; ++jj) {
-      const int j = t0 + c16 + 16 * jj;
-      bool vis = row_ok && j <= my_pos && j < ctx;
-      if (a.window > 0) vis = vis && (j > my_pos - a.window);
-      s[jj] = vis ? fmaf(slope, static_cast<float>(j - my_pos), s[jj] * a.scale) : -INFINITY;
-      tmax = fmaxf(tmax, s[jj]);
-    }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, KVF_WAVE));
-    const float m_new = fmaxf(m_run, tmax);
-    float corr = 1.f, psum = 0.f;
-    if (m_new == -INFINITY) {
-#pragma unroll
-      for (int jj = 0; jj < BKEYS / 16; ++jj) Ps[r][c16 + 16 * jj] = 0.f;
+            for (int x = 0; x < 4; ++x)
+              if (j + x < lo || j + x > hi) v[x] = 0.f;
+          }
+        }
+        *reinterpret_cast<f32x4*>(&KVs[e * VLD + c]) = v;
+      }
     } else {
-      corr = expf(m_run - m_new);  // exp(-inf) = 0 on the first visible tile
-#pragma unroll
-      for (int jj = 0; jj < BKEYS / 16; ++jj) {
-        const float p = expf(s[jj] - m_new);
-        Ps[r][c16 + 16 * jj] = p;
-        psum += p;
+      for (int idx = tid; idx < BK * D; idx += 256) {
+        const int e = idx / BK, c = idx - e * BK;
+        const int j = t0 + c;
+        float v = 0.f;
+        if (j >= lo && j <= hi) {
+          const int blk = j / a.block_size;
+          const int page = blk < a.table_stride ? table[blk] : -1;
+          if (page >= 0 && page < a.num_blocks)
+            v = Elem<T>::load(v_pages + ((static_cast<size_t>(page) * a.KV + kvh) * D + e) * a.block_size +
+                              (j - blk * a.block_size));
+        }
+        KVs[e * VLD + c] = v;
       }
     }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) psum += __shfl_xor(psum, o, KVF_WAVE);
-    l_run = l_run * corr + psum;
-    m_run = m_new;
-#pragma unroll
-    for (int j = 0; j < DMAX / 16; ++j) acc[j] *= corr;
-    // ---- V tile (overwrites the K tile once every thread has finished with it); V pages hold
-    // the keys of one element side by side, so a thread walks keys fastest
     __syncthreads();
-    for (int idx = tid; idx < BKEYS * D; idx += 256) {
-      const int e = idx / BKEYS, c = idx - e * BKEYS;
-      const int j = t0 + c;
-      float v = 0.f;
-      if (j >= lo && j <= hi) {
-        const int blk = j / a.block_size;
-        const int page = blk < a.table_stride ? table[blk] : -1;
-        if (page >= 0 && page < a.num_blocks)
-          v = Elem<T>::load(v_pages + ((static_cast<size_t>(page) * a.KV + kvh) * D + e) * a.block_size +
-                            (j - blk * a.block_size));
+    if (mine) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        if (16 * t >= D) break;
+        f32x4 o = acc[t] * corr;
+#pragma unroll
+        for (int st = 0; st < ST; ++st) {
+          const f32x4 vf = *reinterpret_cast<const f32x4*>(&KVs[(16 * t + j16) * VLD + 16 * st + 4 * g4]);
+#pragma unroll
+          for (int v = 0; v < 4; ++v) o = mfma4(vf[v], p[st][v], o);
+        }
+        acc[t] = o;
       }
-      KVs[c][e] = v;
-    }
-    __syncthreads();
-    for (int c = 0; c < BKEYS; ++c) {
-      const float p = Ps[r][c];
-#pragma unroll
-      for (int j = 0; j < DMAX / 16; ++j)
-        if (c16 + 16 * j < D) acc[j] = fmaf(p, KVs[c][c16 + 16 * j], acc[j]);
     }
   }
   if (!row_ok) return;
-  const int i = my_row / G, g = my_row - i * G;
-  T* o = out + static_cast<size_t>(q0 + i) * a.o_stride + (kvh * G + g) * D;
+  T* o = out + static_cast<size_t>(q0 + tok) * a.o_stride + head * D + 4 * g4;
   const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
 #pragma unroll
-  for (int j = 0; j < DMAX / 16; ++j)
-    if (c16 + 16 * j < D) Elem<T>::store(o + c16 + 16 * j, acc[j] * inv);
+  for (int t = 0; t < DT; ++t)
+    if (16 * t < D) store4(o + 16 * t, acc[t] * inv);
 }
 
 template <typename T>
@@ -187,15 +253,15 @@ int launch(const void* q, const void* k_pages, const void* v_pages, const int* b
            const int* cu_q, const int* ctx_lens, const int* work, int num_work, void* out,
            AttnArgs a, hipStream_t s) {
   if (num_work <= 0) return 0;
-  dim3 grid(num_work, a.KV);
-#define GO(DMAX, BKEYS)                                                                           \
-  hipLaunchKernelGGL((attn_tile_kernel<T, DMAX, BKEYS>), grid, dim3(256), 0, s,                   \
+  dim3 grid(2 * num_work, a.KV);
+#define GO(DMAX)                                                                                  \
+  hipLaunchKernelGGL((attn_mfma32_kernel<T, DMAX>), grid, dim3(256), 0, s,                        \
                      static_cast<const T*>(q), static_cast<const T*>(k_pages),                    \
                      static_cast<const T*>(v_pages), block_table, cu_q, ctx_lens, work,           \
                      static_cast<T*>(out), a)
-  if (a.d <= 64) GO(64, 64);
-  else if (a.d <= 128) GO(128, 64);
-  else GO(256, 32);
+  if (a.d <= 64) GO(64);
+  else if (a.d <= 128) GO(128);
+  else GO(256);
 #undef GO
   return kvf_last_error();
 }
@@ -497,24 +563,24 @@ KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_p
 }
 
 // dtype: 0 = fp32, 1 = bf16.  d must be a multiple of 16 and at most 256 (checked by the caller
-// and here).  tiles_per_seq == 0: `work` holds num_work rows (sequence, 16-row tile, tile or -1).
-// tiles_per_seq > 0: num_work sequences, listed in `work` or 0..num_work-1 when it is null, each
-// with that many tiles (single-token queries need ceil(G / 16)).
+// and here).  `work` holds num_work rows (sequence, item, item or -1), an item being
+// kvf_attn_generic_rows_per_item() rows of (query token, head in the kv head's group).
 KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, const void* v_pages,
                                 const int* block_table, const int* cu_q, const int* ctx_lens,
-                                const int* work, int num_work, int tiles_per_seq, void* out, int H,
-                                int KV, int d, int block_size, int num_blocks, int table_stride,
-                                int q_stride, int o_stride, int window, int n_seqs, float scale,
+                                const int* work, int num_work, void* out, int H, int KV, int d,
+                                int block_size, int num_blocks, int table_stride, int q_stride,
+                                int o_stride, int window, int n_seqs, float scale,
                                 const float* slopes, hipStream_t s) {
-  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || tiles_per_seq < 0 ||
-      (tiles_per_seq == 0 && !work))
+  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || !work || block_size <= 0 ||
+      q_stride % 4 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             tiles_per_seq, scale, slopes};
-  num_work *= tiles_per_seq > 0 ? tiles_per_seq : 2;
+             scale, slopes};
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)
     return launch<bf16_t>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   return static_cast<int>(hipErrorInvalidValue);
 }
+
+KVF_EXPORT int kvf_attn_generic_rows_per_item() { return ITEM_ROWS; }

@@ -1,16 +1,20 @@
-// C[M, N] = A[M, K] * W[N, K]^T with fp32 multiply and fp32 accumulate on the vector ALUs.
+// C[M, N] = A[M, K] * W[N, K]^T with fp32 multiply and fp32 accumulate.
 // This is the matrix product of the true 32-bit path and the fallback for operand types the
-// MFMA kernels do not take (for instance a weight that the checkpoint stores in fp32 while
-// activations are bf16).  No reduced-precision matrix instruction is used.
+// bf16 MFMA kernels do not take (for instance a weight that the checkpoint stores in fp32 while
+// activations are bf16).  No reduced-precision matrix instruction is used: operands stored in
+// bf16 are widened (exactly) before they are multiplied.
 //
-// Two kernels.  Many rows (a portion of a prompt): tiles of 64 x 64 outputs, every output summed
+// Many rows (a portion of a prompt), rows of K that start on 16 bytes: tiles of 128 x 128
+// outputs on the matrix cores with v_mfma_f32_32x32x2_f32, which multiplies and adds in fp32
+// (gemm_mfma32_kernel below).  Many rows otherwise, and kept for comparison: tiles of 64 x 64
+// outputs on the vector ALUs, every output summed
 // over k = 0..K-1 in that order by one thread.  Few rows (decode steps), where the product is
 // bound by reading W once: a wave owns one to four columns of W for all rows, its lanes walk K side by
 // side with 16-byte loads (a wave reads 1 KB of a row of W at a time, several such loads in
 // flight), every lane keeps a partial sum per output and the 64 partial sums are added in a fixed
 // tree at the end.  Within either kernel a row's result does not depend on the number of rows, on
-// the row's place in the batch or on the grid; between the two the order of the sums differs, so
-// results agree to rounding.
+// the row's place in the batch or on the grid; between the kernels the order of the sums differs,
+// so results agree to rounding.
 //
 // Output modes: 0 = store as TO;  1 = add into a fp32 matrix (the residual stream).
 #include "common.h"
@@ -161,6 +165,110 @@ template <> struct Quad<bf16_t> {
   }
 };
 
+// ---- many rows on the matrix cores, true fp32.
+// A workgroup of four waves owns 128 x XN outputs; a wave owns 64 x (XN / 2) of them as 32 x 32
+// tiles of v_mfma_f32_32x32x2_f32 (lane l supplies A[row l % 32][k = l / 32] and
+// W[column l % 32][k = l / 32], and holds 16 outputs of column l % 32).  K is walked in tiles of
+// 32: the tile after the current one travels from memory to registers while the matrix cores work
+// on the current one from LDS.  Within a tile of 32 the two halves of the wave take k = 8u + e
+// and k = 8u + 4 + e in instruction (u, e), so that a lane reads its operands from LDS 16 bytes
+// at a time; the order of the sums is fixed by K alone.  Rows of A and W start on 16 bytes
+// (8 for bf16) and K is a multiple of 4: the caller checks.
+constexpr int XM = 128, XK = 32, XLD = XK + 4;   // LDS rows 144 bytes apart
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+template <typename TA, typename TW, typename TO, int MODE, int XN>
+__global__ __launch_bounds__(256) void gemm_mfma32_kernel(const TA* __restrict__ A,
+                                                          const TW* __restrict__ W,
+                                                          TO* __restrict__ C, int M, int N, int K,
+                                                          int lda, int ldc) {
+  constexpr int CT = XN / 64;          // 32-column tiles per wave
+  constexpr int WQ = XN / 32;          // float4 of W a thread stages per k-tile
+  __shared__ __align__(16) float As[XM][XLD];
+  __shared__ __align__(16) float Ws[XN][XLD];
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE;
+  const int m0 = blockIdx.y * XM, n0 = blockIdx.x * XN;
+  const int wm = (wave / 2) * 64, wn = (wave % 2) * (XN / 2);
+  const int r32 = lane % 32, half = lane / 32;
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  f32x16 acc[2][CT];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < CT; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // what this thread stages: row srow + 32 i, elements skq .. skq + 3 of the k-tile
+  const int srow = tid / 8, skq = (tid % 8) * 4;
+  float4 ra[4], rw[WQ];
+  auto fetch = [&](int k0) {
+    const int k = k0 + skq;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + srow + 32 * i;
+      ra[i] = (m < M && k < K) ? Quad<TA>::load(A + static_cast<size_t>(m) * lda + k) : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < WQ; ++i) {
+      const int n = n0 + srow + 32 * i;
+      rw[i] = (n < N && k < K) ? Quad<TW>::load(W + static_cast<size_t>(n) * K + k) : zero;
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<float4*>(&As[srow + 32 * i][skq]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < WQ; ++i) *reinterpret_cast<float4*>(&Ws[srow + 32 * i][skq]) = rw[i];
+  };
+
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += XK) {
+    __syncthreads();   // the tile before has been read by every wave
+    stage();
+    __syncthreads();
+    if (k0 + XK < K) fetch(k0 + XK);
+#pragma unroll
+    for (int u = 0; u < XK / 8; ++u) {
+      float4 a[2], w[CT];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = *reinterpret_cast<const float4*>(&As[wm + 32 * i + r32][8 * u + 4 * half]);
+#pragma unroll
+      for (int j = 0; j < CT; ++j) w[j] = *reinterpret_cast<const float4*>(&Ws[wn + 32 * j + r32][8 * u + 4 * half]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < CT; ++j) {
+            const float av = e == 0 ? a[i].x : e == 1 ? a[i].y : e == 2 ? a[i].z : a[i].w;
+            const float wv = e == 0 ? w[j].x : e == 1 ? w[j].y : e == 2 ? w[j].z : w[j].w;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, wv, acc[i][j], 0, 0, 0);
+          }
+    }
+  }
+  // output v of a lane: row 8 (v / 4) + 4 (lane / 32) + v % 4 of the tile, column lane % 32
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < CT; ++j) {
+      const int n = n0 + wn + 32 * j + r32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm + 32 * i + 8 * (v / 4) + 4 * half + v % 4;
+        if (m >= M) continue;
+        TO* c = C + static_cast<size_t>(m) * ldc + n;
+        if (MODE == 1) {
+          Elem<TO>::store(c, Elem<TO>::load(c) + acc[i][j][v]);
+        } else {
+          Elem<TO>::store(c, acc[i][j][v]);
+        }
+      }
+    }
+}
+
 // MT rows per workgroup (1, 2, 4, 8 or 16); SN columns of W per wave, each read DEPTH steps
 // ahead, so that SN * DEPTH loads of 16 bytes are in flight per lane: narrow outputs (few
 // columns, hence few waves) take one column per wave and look far ahead, wide ones four columns.
@@ -264,6 +372,20 @@ int launch_stream(const TA* A, const TW* W, TO* C, int M, int N, int K, int lda,
 }
 
 constexpr int STREAM_MAX_M = 32;
+int g_vector_alus_only = 0;   // tests: many rows through the 64 x 64 tiles of the vector ALUs
+
+// Compute units of the current device, asked once per device.
+int compute_units() {
+  static int known[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (known[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    known[dev] = n;
+  }
+  return known[dev];
+}
 
 template <typename TA, typename TW, typename TO, int MODE>
 int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldc,
@@ -289,6 +411,22 @@ int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, 
                        N, K, lda, ldc);
     return kvf_last_error();
   }
+  if (quads && !g_vector_alus_only) {
+    // tiles of 128 columns where they still give every compute unit two workgroups, of 64 else
+    const int wide = ((N + 127) / 128) * ((M + XM - 1) / XM);
+    if (wide >= 2 * compute_units()) {
+      dim3 mgrid((N + 127) / 128, (M + XM - 1) / XM);
+      hipLaunchKernelGGL((gemm_mfma32_kernel<TA, TW, TO, MODE, 128>), mgrid, dim3(256), 0, s,
+                         static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C),
+                         M, N, K, lda, ldc);
+    } else {
+      dim3 mgrid((N + 63) / 64, (M + XM - 1) / XM);
+      hipLaunchKernelGGL((gemm_mfma32_kernel<TA, TW, TO, MODE, 64>), mgrid, dim3(256), 0, s,
+                         static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C),
+                         M, N, K, lda, ldc);
+    }
+    return kvf_last_error();
+  }
   dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   hipLaunchKernelGGL((gemm_tile_kernel<TA, TW, TO, MODE>), grid, dim3(256), 0, s,
                      static_cast<const TA*>(A), static_cast<const TW*>(W), static_cast<TO*>(C), M,
@@ -296,6 +434,14 @@ int launch(const void* A, const void* W, void* C, int M, int N, int K, int lda, 
   return kvf_last_error();
 }
 }  // namespace
+
+// For tests that compare the two many-row kernels: nonzero keeps products of many rows on the
+// vector ALUs.  Returns the setting before.
+KVF_EXPORT int kvf_gemm_generic_vector_alus_only(int on) {
+  const int before = g_vector_alus_only;
+  g_vector_alus_only = on;
+  return before;
+}
 
 // a_type / w_type: 0 = fp32, 1 = bf16.  out_mode: 0 = store in a_type... see table below.
 //   out_kind 0: store fp32      out_kind 1: store bf16      out_kind 2: add into fp32

@@ -459,6 +459,14 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
           m, n, k, lda, ldc, _stream()), "gemm_generic")
 
 
+def gemm_generic_vector_alus_only(on: bool) -> bool:
+    """For tests: keep 32-bit products of many rows on the vector ALUs (the kernel of 64 x 64
+    tiles that the matrix-core kernel replaced) or let them go to the matrix cores again.
+    Returns the setting before."""
+    f = _fn("gemm_generic", "kvf_gemm_generic_vector_alus_only", [c_int])
+    return bool(f(1 if on else 0))
+
+
 def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: float | None = None,
                silu_pairs: bool = False, accumulate: bool = False) -> None:
     """The MFMA weight-streaming product with work folded in at both ends.
@@ -659,7 +667,7 @@ def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int, ro
     size allows them; they pay when the work fills the chip anyway, see ``attn_mfma.hip``)."""
     if attention_on_matrix_cores(dtype, block_size):
         return int(_fn("attn_mfma", "kvf_attn_mfma_rows_per_item", [c_int, c_int])(int(head_dim), int(row_tiles)))
-    return 16
+    return int(_fn("attn_generic", "kvf_attn_generic_rows_per_item", [])())
 
 
 def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -689,23 +697,18 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window),
               n_seqs, float(scale), sl, _stream()), "attn_mfma_prefill")
         return
-    if rows_per_item != 16:
-        raise KernelError("attn_prefill: the vector-ALU kernel takes items of 16 rows")
-    _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, work.shape[0], 0, out,
-                  H, KV, d, scale, window, n_seqs, sl)
-
-
-def _attn_generic(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, tiles_per_seq,
-                  out, H, KV, d, scale, window, n_seqs, slopes_ptr=None) -> None:
-    nb, _, bs, _ = k_pages.shape
+    if rows_per_item != prefill_rows_per_item(q.dtype, d, bs):
+        raise KernelError(f"attn_prefill: the 32-bit kernel takes items of "
+                          f"{prefill_rows_per_item(q.dtype, d, bs)} rows, got {rows_per_item}")
+    if q.stride(0) % 4 or out.stride(0) % 4:
+        raise KernelError("attn_prefill: rows of q and out must start on 16 bytes")
     f = _fn("attn_generic", "kvf_attn_generic",
-            [c_int] + [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 10
+            [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10
             + [c_float, c_void_p, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-          block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(),
-          work.data_ptr() if work is not None else None, num_work, tiles_per_seq, out.data_ptr(),
-          H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs,
-          float(scale), slopes_ptr, _stream()), "attn_generic")
+          block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
+          work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
+          out.stride(0), int(window), n_seqs, float(scale), sl, _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,

@@ -599,6 +599,58 @@ def test_gemm_generic_few_rows_over_long_and_uneven_k(m, tw):
     torch.testing.assert_close(acc.double(), want + 1.0, atol=3e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("ta", DTYPES)
+@pytest.mark.parametrize("tw", DTYPES)
+@pytest.mark.parametrize("mnk", [(33, 130, 96), (200, 70, 260), (129, 257, 2052), (300, 1000, 64),
+                                 (128, 128, 32), (260, 4100, 36)])
+def test_gemm_generic_many_rows_on_the_matrix_cores(ta, tw, mnk):
+    """More than 32 rows with rows of K that start on 16 bytes go to v_mfma_f32_32x32x2_f32:
+    32-bit multiply and add, so 32-bit operands that bfloat16 cannot hold give a 64-bit product's
+    result to 32-bit rounding; tails in M, N and K, tiles of 128 and of 64 columns, both ways of
+    storing and adding into the stream.  A row's result does not depend on the rows around it, and
+    the kernel of the vector ALUs, kept for this comparison, agrees to rounding."""
+    m, n, k = mnk
+    if ta == tw == torch.bfloat16:
+        pytest.skip("bf16 x bf16 with many rows is the library's or the bf16 kernel's product")
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(ta).to(DEV)
+    w = (torch.randn(n, k, generator=g) * 0.1).to(tw).to(DEV)
+    if ta == torch.float32:
+        assert not torch.equal(a.bfloat16().float(), a)
+    want = a.double() @ w.double().T
+    out = torch.full((m, n), 7.0, device=DEV)
+    ops().gemm(a, w, out)
+    torch.testing.assert_close(out.double(), want, atol=2e-5, rtol=1e-5)
+    before = ops().gemm_generic_vector_alus_only(True)
+    try:
+        fma = torch.full((m, n), 7.0, device=DEV)
+        ops().gemm(a, w, fma)
+    finally:
+        ops().gemm_generic_vector_alus_only(before)
+    torch.testing.assert_close(fma.double(), want, atol=2e-5, rtol=1e-5)
+    torch.testing.assert_close(out, fma, atol=2e-5, rtol=1e-5)
+    if k > 64:
+        assert not torch.equal(out, fma)        # another order of summation: it is the other kernel
+    acc = torch.ones(m, n, device=DEV)
+    ops().gemm(a, w, acc, accumulate=True)
+    torch.testing.assert_close(acc.double(), want + 1.0, atol=2e-5, rtol=1e-5)
+    half = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    ops().gemm(a, w, half)
+    torch.testing.assert_close(half.double(), want, atol=2e-2, rtol=2e-2)
+    # the same rows among fewer: the same bits
+    lo = 0 if m < 80 else m // 3
+    hi = min(m, lo + 40)
+    part = torch.empty(hi - lo, n, device=DEV)
+    ops().gemm(a[lo:hi], w, part)
+    assert torch.equal(part, out[lo:hi])
+    # a view with a wider row stride
+    wide = torch.zeros(m, k + 24, dtype=ta, device=DEV)
+    wide[:, :k] = a
+    again = torch.empty(m, n, device=DEV)
+    ops().gemm(wide[:, :k], w, again)
+    assert torch.equal(again, out)
+
+
 @pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
 @pytest.mark.parametrize("n,k", [(6150, 516), (16390, 260)])
 @pytest.mark.parametrize("tw", DTYPES)
@@ -709,7 +761,7 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
     want = attn_reference(paged, q, seq_lens, q_lens, scale, window or None).reshape(n, H * d)
     sizes = sorted({ops().prefill_rows_per_item(dtype, d, bs, tiles) for tiles in (1, 2)})
     assert sizes == ([64, 128] if dtype == torch.bfloat16 and bs % 8 == 0 and d <= 128 else
-                     [64] if dtype == torch.bfloat16 and bs % 8 == 0 else [16])
+                     [64])          # the 32-bit kernel's items: four waves of 16 rows
     for row_tiles, per_item in enumerate(sizes, 1):
         out.zero_()
         ops().attn_prefill(buf.to(DEV), paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV),

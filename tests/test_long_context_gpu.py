@@ -171,7 +171,7 @@ def test_a_run_of_2048_queries_at_the_end_of_32k_keys(d, dtype):
     cu = torch.tensor([0, RUN], dtype=torch.int32, device=DEV)
     ctx = torch.tensor([N], dtype=torch.int32, device=DEV)
     sizes = sorted({ops().prefill_rows_per_item(dtype, d, BS, tiles) for tiles in (1, 2)})
-    assert sizes == ([64, 128] if dtype == torch.bfloat16 else [16])
+    assert sizes == ([64, 128] if dtype == torch.bfloat16 else [64])
     for per_item in sizes:
         for paired in (True, False):
             out = torch.zeros(RUN, H * d, dtype=dtype, device=DEV)
