@@ -12,12 +12,14 @@ N(0, 0.02), batch 8, 512-token uniform-random prompts, greedy, context cap 8192,
 tokens.  A step is one decode step of the whole engine (scheduler, batch building, forward,
 sampling, bookkeeping).  One JSON line is printed; besides the decode figure it carries a
 2,048-token prefill, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
-``points`` also holds (unless ``--no-points``) the same model in true 32-bit (decode at batch 1
+``points`` also holds (unless ``--no-points``) the same model over contexts of 4,096 and 8,192
+tokens (decode at batch 8 and 64, one prompt of 8,192 tokens), the same model in true 32-bit (decode at batch 1
 and 8, prefill of 2,048 tokens, with their shares of the fp32 bounds), the mixed workload at the
 Llama 3.2 3B shape (32 requests, prompts of 128 to 4,096 tokens, chunked prefill under a
 2,048-token budget beside decode steps, 256 new tokens each) and long-context decoding at the
-Llama 3.1 8B shape, all 32 layers (batch 16 at 32,768-token prompts, 128 new tokens); these two
-draw their random weights on the device.
+Llama 3.1 8B shape, all 32 layers (batch 16 at 32,768-token prompts, 128 new tokens; before it
+decode at batch 1 and 8 over 512-token prompts); the 32-bit, 3B and 8B models draw their random
+weights on the device.
 Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
 for fp32.
 """
@@ -242,6 +244,33 @@ def fp32_points(cfg, vocab, nums, steps=48, warmup=8):
     return out
 
 
+def longer_1b_points(folder, vocab, nums, steps=32, warmup=4):
+    """The 1B shape in bf16 further out: decode at batch 8 and 64 over contexts of 4,096 and
+    8,192 tokens (their share of the HBM roofline), and one prompt of 8,192 tokens read in
+    portions of 2,048 (its share of the matrix-core peak)."""
+    import torch
+    out = {}
+    for ctx in (4096, 8192):
+        for b in (8, 64):
+            prompt = ctx - steps - warmup - 8
+            need = b * (prompt + steps + warmup + early_tokens(b, prompt) + 32)
+            engine = build_engine(folder, "bfloat16", b, need, context_cap=ctx + 1024)
+            r = decode_run(engine, vocab, b, prompt, steps, warmup)
+            key = f"decode_b{b}_ctx{ctx}"
+            out[key] = round(r["tok_s"], 1)
+            out[key + "_ms"] = round(r["ms_per_step"], 4)
+            out[key + "_hbm_frac"] = round(
+                decode_bytes(engine, nums, 2, b, r["mean_ctx"]) / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4)
+            if ctx == 8192 and b == 8:
+                s = prefill_run(engine, vocab, 8192, repeats=2)
+                out["prefill_8192_tok_s"] = round(8192 / s, 1)
+                out["prefill_8192_ms"] = round(s * 1e3, 3)
+                out["prefill_8192_frac"] = round(prefill_flops(nums, 8192) / s / MFMA_PEAK["bfloat16"], 4)
+            del engine
+            torch.cuda.empty_cache()
+    return out
+
+
 def mixed_3b_points(requests=32, new_tokens=256):
     """BASELINE's mixed workload at the Llama 3.2 3B shape, bf16."""
     import torch
@@ -278,6 +307,13 @@ def long_8b_points(batch=16, prompt_len=32768, new_tokens=128, warmup=8):
     steps = new_tokens - 1
     need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
     engine = build_engine(cfg, "bfloat16", batch, need, context_cap=prompt_len + 1024)
+    short = {}
+    for b in (1, 8):        # the same model over short contexts: 512-token prompts, batch 1 and 8
+        r = decode_run(engine, cfg["vocab_size"], b, 512, 48, 8)
+        short[f"decode_8b_b{b}"] = round(r["tok_s"], 1)
+        short[f"decode_8b_b{b}_ms"] = round(r["ms_per_step"], 4)
+        short[f"decode_8b_b{b}_hbm_frac"] = round(
+            decode_bytes(engine, nums, 2, b, r["mean_ctx"]) / (r["seconds"] / 48) / 1e9 / HBM_PEAK_GBS, 4)
     t0 = time.perf_counter()
     r = decode_run(engine, cfg["vocab_size"], batch, prompt_len, steps, warmup)
     total = time.perf_counter() - t0
@@ -286,7 +322,8 @@ def long_8b_points(batch=16, prompt_len=32768, new_tokens=128, warmup=8):
            "long_8b_hbm_frac": round(read / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
            "long_8b_layers": cfg["num_hidden_layers"], "long_8b_batch": batch,
            "long_8b_context": int(r["mean_ctx"]), "long_8b_steps": steps,
-           "long_8b_prefill_tok_s": round(batch * prompt_len / max(total - r["seconds"], 1e-9), 1)}
+           "long_8b_prefill_tok_s": round(batch * prompt_len / max(total - r["seconds"], 1e-9), 1),
+           **short}
     del engine
     torch.cuda.empty_cache()
     return out
@@ -356,7 +393,7 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true",
                     help="skip decode at batch 1 and 64, the 32-bit run and the 3B and 8B workloads")
     ap.add_argument("--only-points", default=None,
-                    help="comma-separated subset of fp32,mixed_3b,long_8b to run besides the main line")
+                    help="comma-separated subset of longer_1b,fp32,mixed_3b,long_8b to run besides the main line")
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
@@ -436,8 +473,9 @@ def main() -> int:
             torch.cuda.empty_cache()
         more = {}
         if points and args.preset == "llama-1b" and layers_run == full_layers:
-            chosen = set((args.only_points or "fp32,mixed_3b,long_8b").split(","))
-            for name, fn in (("fp32", lambda: fp32_points(cfg, vocab, nums)),
+            chosen = set((args.only_points or "longer_1b,fp32,mixed_3b,long_8b").split(","))
+            for name, fn in (("longer_1b", lambda: longer_1b_points(folder, vocab, nums)),
+                             ("fp32", lambda: fp32_points(cfg, vocab, nums)),
                              ("mixed_3b", mixed_3b_points), ("long_8b", long_8b_points)):
                 if name not in chosen:
                     continue
