@@ -247,6 +247,39 @@ def test_a_preempted_request_is_fed_again_into_pages_others_have_used(model_a):
     assert engine.cache.num_free_blocks == engine.cache.num_blocks
 
 
+def test_without_chunked_prefill_a_preempted_request_that_outgrew_the_budget_goes_on(model_a):
+    """Chunked prefill off, eight tokens a step, five pages of four: the second of two 7-token
+    prompts loses its pages after it has grown past eight tokens, so what it has to be fed again
+    no longer fits a step.  It is fed in portions (the reference would leave it at the head of
+    the line for ever, src/tokenvault/scheduler.py:109-129 against :206-207), ``generate``
+    returns, and every token of both requests is the plain model's choice."""
+    folder, oracle = model_a
+    prompts = [[9, 200, 31, 77, 5, 150, 42], [120, 8, 66, 201, 13, 90, 3]]
+    cfg = EngineConfig(cache=CacheConfig(block_size=4, num_blocks=5),
+                       scheduler=SchedulerConfig(max_num_seqs=2, max_num_batched_tokens=8,
+                                                 enable_chunked_prefill=False),
+                       dtype="float32", decode_run_steps=1)
+    engine = InferenceEngine.from_folder(folder, cfg)
+    outs = engine.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0))
+    assert engine.scheduler.num_preemptions >= 1 and max(engine.metrics.batched_tokens) <= 8
+    assert [len(o.output_token_ids) for o in outs] == [12, 12]
+    for p, o in zip(prompts, outs):
+        oracle.check_choices(p, o.output_token_ids, 1e-4)
+        want, gaps = oracle.greedy(p, 12)
+        assert_greedy_equal(o.output_token_ids, want, gaps)
+    assert engine.cache.num_free_blocks == engine.cache.num_blocks
+
+
+def test_generate_raises_when_nothing_can_be_planned(model_a, monkeypatch):
+    """A scheduler that plans nothing while requests wait would make ``generate`` ask for ever;
+    it raises instead (forced here by a scheduler that refuses to admit)."""
+    folder, _ = model_a
+    engine = engine_for(folder)
+    monkeypatch.setattr(engine.scheduler, "_admit", lambda plan, budget: None)
+    with pytest.raises(RuntimeError, match="stuck"):
+        engine.generate([[5, 17, 3]], GREEDY)
+
+
 @pytest.mark.parametrize("budget", [16, 24])
 def test_chunked_prefill_preserves_outputs(model_a, budget):
     folder, oracle = model_a
