@@ -140,6 +140,10 @@ class MetaBuffers:
         for w in self.table_widths:
             self.table_off.append(off)
             off += max_seqs * w
+        # room behind the batch's own fields for what parts send along with a step
+        # (``Step.upload_ints``)
+        self.extra_off, self.extra_size = off, max(4096, 4 * max_tokens)
+        off += self.extra_size
         self.total = off
         self.device_buf = torch.zeros(self.total, dtype=torch.int32, device=device)
         pin = torch.device(device).type == "cuda"
@@ -193,6 +197,28 @@ class Step:
         # library product over many rows leaves it here instead of running an add kernel; the
         # next norm adds it on its way (``take_owed``), anything else calls ``settle`` first.
         self.owed: tuple[torch.Tensor, torch.Tensor] | None = None
+        # the staging memory this step was filled from (``fill_step``), for ``upload_ints``
+        self._meta: "MetaBuffers | None" = None
+        self._turn = 0
+        self._extra_used = 0
+
+    def upload_ints(self, values) -> torch.Tensor:
+        """An int32 device tensor holding ``values`` (a flat sequence or array), for what a part
+        derives on the host for this step (a work list, a table): it travels through the same
+        pinned staging memory as the batch itself, queued on the stream without waiting for
+        the device, and stays valid until the next step is filled.  A step that was not filled
+        from staging memory (or has no room left there) sends it the slow way."""
+        arr = np.asarray(values, dtype=np.int32).reshape(-1)
+        meta, n = self._meta, int(arr.shape[0])
+        if meta is None or not meta.device_buf.is_cuda or self._extra_used + n > meta.extra_size:
+            return torch.from_numpy(arr.copy()).to(self.device)
+        lo = meta.extra_off + self._extra_used
+        self._extra_used += (n + 3) // 4 * 4
+        meta.staging_np[self._turn][lo:lo + n] = arr
+        dst = meta.device_buf[lo:lo + n]
+        dst.copy_(meta.staging[self._turn][lo:lo + n], non_blocking=True)
+        meta.events[self._turn].record()     # the staging memory is free again after this copy
+        return dst
 
     def owe(self, residual: torch.Tensor, product: torch.Tensor) -> None:
         self.settle()
@@ -374,4 +400,5 @@ def fill_step(step: Step, meta: MetaBuffers, entries: Sequence[StepEntry], table
     step.decode_shape = DecodeShape(len(live), max(live, default=0), sum(live))
     step.max_position = int(ctx.max()) if Bp else 0
     step.scratch = {}
+    step._meta, step._turn, step._extra_used = meta, turn, 0
     return counts

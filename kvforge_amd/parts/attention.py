@@ -203,7 +203,7 @@ class PagedAttention(Mixer):
             if len(rows) * self.KV < 2 * compute_units(step.device):
                 per_item = ops.prefill_rows_per_item(act, self.d, block_size, 1)
                 rows = prefill_work_rows(step.q_lens, step.prefill_seqs, G, per_item, step.start_pos)
-            found = (torch.tensor(rows, dtype=torch.int32).reshape(-1, 3).to(step.device), per_item)
+            found = (step.upload_ints([x for row in rows for x in row]).view(-1, 3), per_item)
             step.scratch[key] = found
         return found
 

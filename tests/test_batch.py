@@ -189,3 +189,15 @@ def test_uneven_contexts_ask_for_cuts_of_the_key_range():
     assert full.launch_key(DecodeShape(8, 511, 8 * 500)) == (0, 1)
     assert full.launch_key(DecodeShape(32, 32768, 32768 + 31 * 600)) == (64, 8)
     assert windowed.launch_key(DecodeShape(32, 32768, 32768 + 31 * 600)) == (1, 1)
+
+
+def test_what_a_part_sends_along_with_a_step():
+    """``Step.upload_ints``: on the CPU (no staging memory to go through) the values simply
+    become a tensor on the step's device; a step that was never filled does the same."""
+    cache, meta, step = setup()
+    assert step.upload_ints([3, 1, 4]).tolist() == [3, 1, 4]
+    cache.allocate("a", 6)
+    fill_step(step, meta, [StepEntry("a", [1, 2, 3], 3, "last")], cache.block_table, lambda r: -1, 4)
+    got = step.upload_ints([(0, 1, -1), (0, 0, 2)])
+    assert got.dtype == torch.int32 and got.tolist() == [0, 1, -1, 0, 0, 2]
+    assert meta.total == meta.extra_off + meta.extra_size and meta.extra_size >= 4 * 64

@@ -383,3 +383,24 @@ def test_run_order_is_checked():
     spec.schedule = [LayerCall(5)]
     with pytest.raises(ValueError, match="outside"):
         Transformer(spec, torch.float32, DEV)
+
+
+def test_ints_sent_along_with_a_step_arrive_in_stream_order():
+    """``Step.upload_ints`` on the device: several lists in one step land behind each other in
+    the step's own memory, a list too long for it goes the slow way, and the next step may
+    overwrite them only behind this step's work in stream order."""
+    cache = CacheManager(4, [CacheGroup((0,))], 16)
+    cache.allocate("r", 12)
+    step = make_step([StepEntry("r", [0] * 12, 0, "none")], cache, torch.float32)
+    a = step.upload_ints(list(range(10)))
+    b = step.upload_ints([(7, 8, -1), (9, 10, 11)])
+    big = step.upload_ints(list(range(5000)))
+    torch.cuda.synchronize()
+    assert a.tolist() == list(range(10)) and b.tolist() == [7, 8, -1, 9, 10, 11]
+    assert big.tolist() == list(range(5000)) and a.is_cuda and a.dtype == torch.int32
+    assert a.data_ptr() != b.data_ptr() and b.data_ptr() % 16 == 0
+    kept = a.clone()                     # queued before the next step's fill
+    again = make_step([StepEntry("r", [0] * 12, 0, "none")], cache, torch.float32)
+    c = again.upload_ints([5] * 10)
+    torch.cuda.synchronize()
+    assert kept.tolist() == list(range(10)) and c.tolist() == [5] * 10
