@@ -141,7 +141,21 @@ class PagedAttention(Mixer):
             perm[2 * i], perm[2 * i + 1] = i, i + rot // 2
         return perm
 
+    def after_projection(self, qkv: torch.Tensor, step) -> None:
+        """A place for a variant to change the projected rows before they are rotated and
+        written to the cache (a bias on the projections, a norm per head of q and k): ``qkv``
+        is ``[N, (H + 2 KV) d]`` in the step's activation type, q heads, then k heads, then v
+        heads, each head's rotary pairs as neighbouring elements (``pair_permutation``); it is
+        changed in place.  The default does nothing.  A subclass that overrides it runs
+        projection, this, and rotation + cache write as kernels of their own in every step
+        (the kernel that fuses the three has no place for it) and keeps its norm a kernel."""
+
+    def _hooked(self) -> bool:
+        return type(self).after_projection is not PagedAttention.after_projection
+
     def absorb_norm(self, norm) -> bool:
+        if self._hooked():
+            return False
         if self.norm_eps is not None or not getattr(norm, "foldable_into", lambda m: False)(self.w_qkv):
             return False
         self.w_qkv = (self.w_qkv.float() * norm.weight.float()[None, :]).to(torch.bfloat16).contiguous()
@@ -223,7 +237,7 @@ class PagedAttention(Mixer):
             normed = ws.buf("normed", (n, self.hidden), act)
             ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
-        fused = (ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
+        fused = (not self._hooked() and ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
                  and layer.k_pages.dtype == torch.bfloat16)
         if fused and rms is not None:
             # what the layer before owes the stream in fp32 rides in this projection's loads and
@@ -243,6 +257,7 @@ class PagedAttention(Mixer):
         else:
             qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), act)
             ops.gemm(x, self.w_qkv, qkv)
+            self.after_projection(qkv, step)
             ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
                              layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache)
         out = ws.buf("attn_out", (n, H * d), act)

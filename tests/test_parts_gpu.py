@@ -169,6 +169,85 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs, small_chip, m
         torch.testing.assert_close(torch.cat(got[rid]), want[rid], **tol(dtype))
 
 
+class ToyQKNormAttention(PagedAttention):
+    """Attention with a bias on the q projection and an RMS norm per head of q and of k before
+    the rotation, added from here through ``after_projection``: the framework's files know of
+    neither.  The norm's weights are constants of the part (no tensors), one per element."""
+
+    replayable = True
+
+    def __init__(self, *args, q_bias=None, **kw):
+        super().__init__(*args, **kw)
+        self.q_bias = q_bias                           # [H * d], checkpoint order
+        g = torch.Generator().manual_seed(99)
+        self.qk_weight = 1 + 0.2 * torch.randn(self.d, generator=g)      # checkpoint order
+
+    def after_projection(self, qkv, step):
+        H, KV, d = self.H, self.KV, self.d
+        perm = self.pair_permutation().to(qkv.device)   # the part's layout: perm[new] = old
+        w = self.qk_weight.to(qkv.device)[perm]
+        q = qkv[:, :H * d].float().view(-1, H, d)
+        if self.q_bias is not None:
+            q = q + self.q_bias.to(qkv.device).view(H, d)[:, perm]
+        k = qkv[:, H * d:(H + KV) * d].float().view(-1, KV, d)
+        for t, lo in ((q, 0), (k, H * d)):
+            normed = t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+            qkv[:, lo:lo + normed.shape[1] * d] = normed.reshape(normed.shape[0], -1).to(qkv.dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_variant_of_attention_changes_q_and_k_before_the_rotation(dtype):
+    """``PagedAttention.after_projection``: a subclass defined here adds a bias to q and norms
+    every head of q and k; fed in portions and token by token it gives what the same
+    computation gives over the whole sequence, and without the hook's work the result is
+    another one."""
+    H, KV, d, hidden, bs = 4, 2, 32, 40, 8
+    rot = RotaryPositions(d, 1000.0)
+    rot.prepare(64, DEV)
+    bias = rand(H * d, seed=31, scale=0.5)
+    part = ToyQKNormAttention("a", hidden, H, KV, d, rot, q_bias=bias)
+    assert not part.absorb_norm(RMSNorm("n", hidden, 1e-5))
+    w = {"a.q_proj.weight": rand(H * d, hidden, seed=10, scale=0.25).to(dtype),
+         "a.k_proj.weight": rand(KV * d, hidden, seed=11, scale=0.25).to(dtype),
+         "a.v_proj.weight": rand(KV * d, hidden, seed=12, scale=0.15).to(dtype),
+         "a.o_proj.weight": rand(hidden, H * d, seed=13, scale=0.1).to(dtype)}
+    part.load({k: v.to(DEV) for k, v in w.items()})
+    part.seal()
+    x = rand(25, hidden, seed=14).to(dtype)
+    wf = {k: v.float() for k, v in w.items()}
+    T = x.shape[0]
+    cos, sin = plain.rope_cos_sin(torch.arange(T), plain.rope_inv_freq(d, 1000.0))
+
+    def whole(with_hook):
+        q = (x.float() @ wf["a.q_proj.weight"].T).view(T, H, d)
+        k = (x.float() @ wf["a.k_proj.weight"].T).view(T, KV, d)
+        v = (x.float() @ wf["a.v_proj.weight"].T).view(T, KV, d)
+        if with_hook:
+            q = q + bias.view(H, d)
+            q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6) * part.qk_weight
+            k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6) * part.qk_weight
+        q, k = plain.apply_rope(q, cos, sin), plain.apply_rope(k, cos, sin)
+        att = plain.causal_attention(q, k, v, 1 / math.sqrt(d))
+        return att.reshape(T, H * d) @ wf["a.o_proj.weight"].T
+
+    want = whole(True)
+    assert float((want - whole(False)).abs().max()) > 0.05
+    cache = CacheManager(bs, [CacheGroup((0,), attention_pages(KV, d), None)], 8)
+    ls = LayerState(group=0, owns_cache=True,
+                    pages={"k": torch.zeros(8, KV, bs, d, dtype=dtype, device=DEV),
+                           "v": torch.zeros(8, KV, d, bs, dtype=dtype, device=DEV)})
+    cache.allocate("s", 0)
+    got = []
+    for a, b in ((0, 11), (11, 22), (22, 23), (23, 24), (24, 25)):
+        cache.append_slots("s", b, a)
+        step = make_step([StepEntry("s", [0] * (b - a), a, "none")], cache, dtype)
+        residual = torch.zeros(b - a, hidden, device=DEV)
+        part.forward(x[a:b].to(DEV), step, ls, residual)
+        step.settle()
+        got.append(residual.cpu())
+    torch.testing.assert_close(torch.cat(got), want, **tol(dtype))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n", [7, 23])  # few rows: sums in the product kernels; many: owed to the stream
 def test_pre_norm_block(dtype, n):
