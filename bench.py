@@ -272,7 +272,8 @@ def longer_1b_points(folder, vocab, nums, steps=32, warmup=4):
 
 
 def mixed_3b_points(requests=32, new_tokens=256):
-    """BASELINE's mixed workload at the Llama 3.2 3B shape, bf16."""
+    """The mixed workload at the Llama 3.2 3B shape, bf16: 32 requests with prompts of 128 to 4,096
+    tokens, chunked prefill under a 2,048-token budget, 256 decoded tokens each."""
     import torch
     import kvforge_amd
     cfg = kvforge_amd.preset_dict("llama-3b")
@@ -299,7 +300,8 @@ def mixed_3b_points(requests=32, new_tokens=256):
 
 
 def long_8b_points(batch=16, prompt_len=32768, new_tokens=128, warmup=8):
-    """BASELINE's long-context decode at the Llama 3.1 8B shape, all 32 layers, bf16."""
+    """Long-context decode at the Llama 3.1 8B shape, all 32 layers, bf16: batch 16 at prompts of
+    32,768 tokens, 128 new tokens each; before it decode at batch 1 and 8 over short prompts."""
     import torch
     import kvforge_amd
     cfg = kvforge_amd.preset_dict("llama-8b")
