@@ -59,6 +59,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 struct MArgs {
   int H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits;
+  int kv_fastest;  // query runs: the kv head is the grid's fastest index (see kvf_attn_mfma_prefill)
   float scale;
   unsigned bs_magic;  // floor(2^32 / bs) + 1: key / bs == mulhi(key, bs_magic) while key * bs < 2^32
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
@@ -300,6 +301,10 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   constexpr int DC = (DT + 1) / 2;
   constexpr int N_K = 2 * DC, N_FRAG = N_K + DT;          // fragments of a key block
   constexpr int FPW = (N_FRAG + WAVES - 1) / WAVES;       // fragments a wave stages per block
+  // Fragments asked for two blocks ahead (two sets of staging registers) where the registers
+  // that takes do not cost a wave per SIMD: measured at head size 128 with one row tile, 2,048
+  // queries take 75.7 us with one set (three waves per SIMD) and 87.8 with two (two waves).
+  constexpr bool DEEP = RT == 2 || DT <= 4;
   extern __shared__ uint4 frag_lds[];                     // SHARE: [2][N_FRAG][64]
 
   const int lane = threadIdx.x % KVF_WAVE;
@@ -309,7 +314,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   // A work row names a sequence and up to two of its items (the second may be -1), which the
   // workgroup takes one after the other: the host pairs an early item (few keys to walk) with a
   // late one (many), so that under the causal mask all workgroups have about the same to do.
-  const int seq = work[3 * blockIdx.x], kvh = blockIdx.y;
+  const int wrow = a.kv_fastest ? blockIdx.y : blockIdx.x, kvh = a.kv_fastest ? blockIdx.x : blockIdx.y;
+  const int seq = work[3 * wrow];
   if (seq < 0 || seq >= a.n_seqs) return;
   const int q0 = cu_q[seq], qlen = cu_q[seq + 1] - q0, ctx = ctx_lens[seq];
   const int start = ctx - qlen;
@@ -317,7 +323,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   const Pages pg{k_pages, vt_pages, block_table + static_cast<size_t>(seq) * a.table_stride, kvh, ctx,
                  j16, kg};
   for (int part = 0; part < 2; ++part) {
-  const int item = work[3 * blockIdx.x + 1 + part];
+  const int item = work[3 * wrow + 1 + part];
   if (item < 0) continue;
   const int wg_tile = item * WAVES * RT;
 
@@ -355,13 +361,23 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   if (SHARE) {
     // fragment f of a block: K (tile f / DC, step f % DC) for f < N_K, then V^T element tiles;
     // wave w stages fragments w, w + 4, ...
-    const int kb_first = (lo_g / 32) * 32;
     // What does not change from block to block is worked out once per fragment: the key a lane
     // reads relative to the block's start, and its offset inside a page apart from the key's slot
     // (in fragments of 16 bytes).
-    uint4 stage[FPW];
-    PageRef page[FPW];
-    int live[FPW];
+    // Two sets of staging registers and of page lookups, named apart (an index chosen at run
+    // time would put them in scratch memory).  While the waves work on block p from LDS, the
+    // fragments of block p + 1 are on their way in one set (asked for a whole block ago, put
+    // into LDS at the end of this one), those of block p + 2 are asked for into the other, and
+    // the pages of block p + 3 are looked up.  Lookups are issued before the fragment loads of
+    // the same block: the load counter runs in order, so waiting for a lookup then does not
+    // also wait for fragments that were asked for after it.
+    struct Stage {
+      uint4 frag[FPW];
+      int live[FPW];
+    };
+    struct Lookup {
+      PageRef page[FPW];
+    };
     int key_off[FPW];
     unsigned lane_off[FPW];
     bool is_k[FPW], whole[FPW];
@@ -381,47 +397,33 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         lane_off[i] = (static_cast<unsigned>(kvh) * D + (f - N_K) * 16 + j16) * (a.bs / 8);
       }
     }
-    auto locate = [&](int kb) {
+    // Every load below reads a valid address whatever the block (a key past the context reads
+    // the table's last entry and page 0, and counts for nothing), so none of them sits in a
+    // branch and the compiler can count them.
+    auto locate = [&](int kb, Lookup& l) {
 #pragma unroll
-      for (int i = 0; i < FPW; ++i) page[i] = page_of_key(pg, a, kb + key_off[i]);
+      for (int i = 0; i < FPW; ++i) l.page[i] = page_of_key(pg, a, kb + key_off[i]);
     };
-    auto fetch = [&](int kb) {
+    auto fetch = [&](int kb, const Lookup& l, Stage& st) {
 #pragma unroll
       for (int i = 0; i < FPW; ++i) {
         const int key = kb + key_off[i];
         const unsigned slot = static_cast<unsigned>(key - block_of(a, key) * a.bs);
-        const bool ok = page[i].ok(a.nb) && whole[i];
-        live[i] = !ok ? 0 : is_k[i] ? 8 : min(ctx - key, 8);
-        const unsigned off = __umul24(ok ? page[i].page : 0, page_stride) + lane_off[i] +
+        const bool ok = l.page[i].ok(a.nb) && whole[i];
+        st.live[i] = !ok ? 0 : is_k[i] ? 8 : min(ctx - key, 8);
+        const unsigned off = __umul24(ok ? l.page[i].page : 0, page_stride) + lane_off[i] +
                              (is_k[i] ? __umul24(slot, D / 8) : slot >> 3);
-        stage[i] = ld16((is_k[i] ? k_pages : vt_pages) + static_cast<size_t>(off) * 8);
+        st.frag[i] = ld16((is_k[i] ? k_pages : vt_pages) + static_cast<size_t>(off) * 8);
       }
     };
-    auto put = [&](int buf) {
+    auto put = [&](int buf, const Stage& st) {
 #pragma unroll
       for (int i = 0; i < FPW; ++i) {
         const int f = wave + i * WAVES;
-        if (f < N_FRAG) frag_lds[(buf * N_FRAG + f) * KVF_WAVE + lane] = keep_first(stage[i], live[i]);
+        if (f < N_FRAG) frag_lds[(buf * N_FRAG + f) * KVF_WAVE + lane] = keep_first(st.frag[i], st.live[i]);
       }
     };
-    if (kb_first <= hi_g) {
-      locate(kb_first);
-      fetch(kb_first);
-      locate(kb_first + 32);
-      put(0);
-    }
-    // Everything loaded so far (the query fragments among it) has to be there before the loop:
-    // otherwise the compiler, not knowing how many loads a first pass through the loop still has
-    // ahead of them, waits for all loads before the first product of every pass.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    int buf = 0;
-    for (int kb = kb_first; kb <= hi_g; kb += 32) {
-      const bool more = kb + 32 <= hi_g;
-      if (more) {
-        fetch(kb + 32);   // its pages were looked up a block ago
-        locate(kb + 64);  // nothing past the context is looked up
-      }
+    auto work_on = [&](int kb, int buf) {
       if (kb <= hi_w && kb + 31 >= lo_w) {
         bf16x8 kf[2][DC], vf[DT];
 #pragma unroll
@@ -434,9 +436,61 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         const bool edge = kb + 31 > pos_min || kb + 32 > ctx || a.window > 0;
         block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
       }
-      if (more) put(buf ^ 1);
+    };
+    const int kb_first = (lo_g / 32) * 32;
+    Stage sa;
+    Lookup la;
+    if constexpr (DEEP) {
+      Stage sb;
+      Lookup lb;
+      if (kb_first <= hi_g) {
+        locate(kb_first, la);
+        locate(kb_first + 32, lb);
+        fetch(kb_first, la, sa);
+        locate(kb_first + 64, la);
+        fetch(kb_first + 32, lb, sb);
+        put(0, sa);
+      }
+      // Everything loaded so far (the query fragments among it) has to be there before the loop:
+      // otherwise the compiler, not knowing how many loads a first pass through the loop still
+      // has ahead of them, waits for all loads before the first product of every pass.
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       __syncthreads();
-      buf ^= 1;
+      // at the top of a pass: LDS half 0 holds block kb, `sb` block kb + 32, `la` the pages of
+      // block kb + 64
+      for (int kb = kb_first; kb <= hi_g; kb += 64) {
+        locate(kb + 96, lb);
+        fetch(kb + 64, la, sa);
+        work_on(kb, 0);
+        put(1, sb);
+        __syncthreads();
+        if (kb + 32 > hi_g) break;
+        locate(kb + 128, la);
+        fetch(kb + 96, lb, sb);
+        work_on(kb + 32, 1);
+        put(0, sa);
+        __syncthreads();
+      }
+    } else {
+      // one set: the fragments of block p + 1 are asked for at the top of block p and put into
+      // LDS at its end; the pages of block p + 2 are looked up meanwhile
+      if (kb_first <= hi_g) {
+        locate(kb_first, la);
+        fetch(kb_first, la, sa);
+        locate(kb_first + 32, la);
+        put(0, sa);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), as above
+      __syncthreads();
+      int buf = 0;
+      for (int kb = kb_first; kb <= hi_g; kb += 32) {
+        fetch(kb + 32, la, sa);
+        locate(kb + 64, la);
+        work_on(kb, buf);
+        put(buf ^ 1, sa);
+        __syncthreads();
+        buf ^= 1;
+      }
     }
   } else {
     PageRef pk[2] = {k_page(pg, a, (lo_w / 32) * 32, 0), k_page(pg, a, (lo_w / 32) * 32, 1)};
@@ -713,8 +767,9 @@ unsigned magic_of(int bs) { return static_cast<unsigned>((1ull << 32) / bs) + 1u
 // Row tiles per wave and LDS sharing by head size: what fits the registers and 64 KB of LDS.
 // One tile per wave keeps more workgroups in flight; two halve what a key block costs per row
 // (looking its pages up, staging it, the barrier) and pay when the work fills the chip anyway
-// (measured at 32 heads of size 64: 8,192 tokens 525 to 441 us; 2,048 tokens 57 to 55; four
-// prompts of 512, 19.9 to 20.7): the caller chooses by the rows it has.
+// (measured at 32 heads of size 64, one item per workgroup: 8,192 tokens 444 to 385 us, 4,096
+// tokens 143 to 114; 2,048 tokens 47 to 54 the other way): the caller chooses by the rows it
+// has and by kvf_attn_mfma_prefill_blocks_per_cu.
 constexpr int runs_max_rt(int dt) { return dt <= 8 ? 2 : 1; }
 constexpr bool runs_share(int dt) { return dt <= 12; }
 
@@ -790,13 +845,42 @@ void launch_split(dim3 grid, hipStream_t s, const void* q, const void* k_pages, 
   X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14) X(15) X(16)
 }  // namespace
 
-// Rows of a query run one workgroup takes with `row_tiles` (1 or 2) tiles per wave, where the
-// head size allows so many: 4 waves x tiles x 16 rows.
 // For measurements: waves per workgroup of the kernel for single tokens (4, 8; 0 = by the grid).
 KVF_EXPORT void kvf_attn_mfma_set_split_waves(int waves) { g_split_waves = waves; }
+// Rows of a query run one workgroup takes with `row_tiles` (1 or 2) tiles per wave, where the
+// head size allows so many: 4 waves x tiles x 16 rows.
 KVF_EXPORT int kvf_attn_mfma_rows_per_item(int d, int row_tiles) {
   const int most = d > 0 && d <= 128 ? 2 : 1;   // runs_max_rt(d / 16)
   return WAVES * (row_tiles >= 2 ? most : 1) * 16;
+}
+
+// Workgroups of the kernel for query runs that a compute unit holds at once, by its registers
+// and LDS: what a caller weighs rows per item against (0 if the head size is not taken).
+template <int DT, int RT>
+int runs_blocks_per_cu() {
+  constexpr bool SHARE = runs_share(DT);
+  constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
+  const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attn_mfma_runs_kernel<DT, RT, SHARE, false>, 256, lds) !=
+      hipSuccess)
+    return 0;
+  return n;
+}
+KVF_EXPORT int kvf_attn_mfma_prefill_blocks_per_cu(int d, int row_tiles) {
+  if (d <= 0 || d % 16 != 0 || d > 256) return 0;
+  const bool two = row_tiles >= 2 && d <= 128;
+  switch (d / 16) {
+#define GO(DT)                                                              \
+  case DT:                                                                  \
+    if constexpr (runs_max_rt(DT) >= 2) {                                   \
+      if (two) return runs_blocks_per_cu<DT, 2>();                          \
+    }                                                                       \
+    return runs_blocks_per_cu<DT, 1>();
+    KVF_EACH_DT(GO)
+#undef GO
+  }
+  return 0;
 }
 
 // Query runs: `work` holds num_work rows (sequence, item, item or -1) where item i covers rows
@@ -813,8 +897,12 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
     return static_cast<int>(hipErrorInvalidValue);
   const int row_tiles = rows_per_item / (WAVES * 16);
   if (rows_per_item != kvf_attn_mfma_rows_per_item(d, row_tiles)) return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, scale, magic_of(bs), slopes};
-  const dim3 grid(num_work, KV);
+  // The kv heads are the fastest index of the grid where the grid allows it: consecutive
+  // workgroups go to consecutive XCDs, so with eight kv heads every XCD walks the keys and values
+  // of one head and finds them in its own L2 after the first workgroup has brought them in.
+  const int kv_fastest = num_work <= 65535 ? 1 : 0;
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, kv_fastest, scale, magic_of(bs), slopes};
+  const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
   case DT: launch_runs<DT>(row_tiles, grid, s, q, k_pages, vt_pages, block_table, work, cu_q, ctx_lens, out, a); break;
@@ -838,7 +926,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, scale, magic_of(bs), slopes};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, 0, scale, magic_of(bs), slopes};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);

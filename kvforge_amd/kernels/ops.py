@@ -670,6 +670,22 @@ def prefill_rows_per_item(dtype: torch.dtype, head_dim: int, block_size: int, ro
     return int(_fn("attn_generic", "kvf_attn_generic_rows_per_item", [])())
 
 
+_blocks_per_cu: dict[tuple, int] = {}
+
+
+def prefill_blocks_per_cu(dtype: torch.dtype, head_dim: int, block_size: int, row_tiles: int = 1) -> int:
+    """Workgroups of the kernel for query runs that one compute unit holds at a time (by its
+    registers and LDS, asked of the runtime once): what fills the chip is this many times the
+    compute units."""
+    key = (dtype, int(head_dim), int(block_size) % 8 == 0, int(row_tiles))
+    if key not in _blocks_per_cu:
+        n = 4
+        if attention_on_matrix_cores(dtype, block_size):
+            n = int(_fn("attn_mfma", "kvf_attn_mfma_prefill_blocks_per_cu", [c_int, c_int])(int(head_dim), int(row_tiles)))
+        _blocks_per_cu[key] = max(1, n)
+    return _blocks_per_cu[key]
+
+
 def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,

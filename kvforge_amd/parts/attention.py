@@ -52,25 +52,23 @@ def skew_cuts(max_ctx: int, sum_ctx: int, n: int) -> int:
 
 def prefill_work_rows(q_lens, prefill_seqs, group_size: int, rows_per_item: int,
                       start_pos=None) -> list[tuple]:
-    """Rows (sequence row, item, item or -1) for every query run longer than one token: a run of
-    ``q`` tokens has ``q * group_size`` rows per kv head, an item covers ``rows_per_item`` of
-    them, and a workgroup takes the items of one row one after the other.  Item ``i`` is paired
-    with item ``n - 1 - i``: under the causal mask the early one walks few keys and the late one
-    many, so every pair has about the same to do.  A run that starts at least half its own length
-    into its sequence (``start_pos``: the keys before each run) is not paired: its items differ
-    by less than that in the keys they walk, and one item per workgroup, the longest walks
-    first, gives twice the workgroups (measured at 32 heads of size 128 with two row tiles per
-    wave: 2,048 queries at the end of 32,768 keys take 2.15 ms in pairs and 1.41 ms alone, at
-    the end of 3,072 keys 148 and 141 us; 512 queries at the end of 32,768 keys, one row tile,
-    1.90 and 0.96 ms)."""
+    """Rows (sequence row, item, -1) for every query run longer than one token: a run of ``q``
+    tokens has ``q * group_size`` rows per kv head, an item covers ``rows_per_item`` of them, and
+    a workgroup takes one item.  Under the causal mask an item walks the keys up to its last
+    row's position (``start_pos``: the keys before each run): the items of all runs are handed
+    out longest walk first, so that the short ones fill the gaps the long ones leave as compute
+    units come free.  (The kernels also take two items per row, an early one paired with a late
+    one, which balances the workgroups among themselves; measured once the kv heads were spread
+    over the XCDs it lost to this order, which keeps twice the workgroups in flight: 2,048
+    queries of 32 heads of size 64 take 58 us in pairs and 47 us one by one, 2,048 at the end
+    of 8,192 keys 398 and 301.)"""
     rows = []
     for b in prefill_seqs:
         n = -(-q_lens[b] * group_size // rows_per_item)
-        if start_pos is not None and 2 * start_pos[b] >= q_lens[b]:
-            rows += [(b, i, -1) for i in reversed(range(n))]
-        else:
-            rows += [(b, i, n - 1 - i if n - 1 - i > i else -1) for i in range((n + 1) // 2)]
-    return rows
+        before = start_pos[b] if start_pos is not None else 0
+        rows += [(before + min(q_lens[b], -(-(i + 1) * rows_per_item // group_size)), b, i) for i in range(n)]
+    rows.sort(key=lambda r: -r[0])        # stable: equal walks stay in sequence and item order
+    return [(b, i, -1) for _, b, i in rows]
 
 
 @register_mixer("attention")
@@ -203,18 +201,29 @@ class PagedAttention(Mixer):
 
     def _prefill_work(self, step, act: torch.dtype, block_size: int):
         """(work rows on the device, rows per item) of the step's query runs, or ``(None, 0)``.
-        Items of two row tiles per wave where the kernel has them and the step's runs then still
-        give every compute unit two workgroups; the layers of a model that agree on group size
-        and item share the rows through the step's scratch."""
+        Items of two row tiles per wave halve what a key block costs per row (its page lookups,
+        staging and barrier) and halve the workgroups.  They are taken where the kernel has them
+        and their workgroups alone are as many as the chip holds of the one-tile kernel at a
+        time (so that short items are left to fill in behind the long ones), or give every
+        compute unit two while every run starts at least its own length into its sequence (then
+        all items walk long and nothing needs filling in).  Measured at 32 heads over 8 kv heads,
+        one against two tiles: 2,048 queries from position 0, 47 against 55 us at head size 64
+        and 70 against 82 at 128; 4,096 queries, 140 against 114 and 231 against 196; 2,048
+        queries behind 2,048 keys, 106 against 100 and 209 against 151.  The layers of a model
+        that agree on group size and item share the rows through the step's scratch."""
         if not step.prefill_seqs:
             return None, 0
         G = self.H // self.KV
         key = ("attention.prefill_work", G, self.KV, self.d, act, block_size)
         found = step.scratch.get(key)
         if found is None:
+            units = compute_units(step.device)
             per_item = ops.prefill_rows_per_item(act, self.d, block_size, 2)
             rows = prefill_work_rows(step.q_lens, step.prefill_seqs, G, per_item, step.start_pos)
-            if len(rows) * self.KV < 2 * compute_units(step.device):
+            groups = len(rows) * self.KV
+            fills = groups >= ops.prefill_blocks_per_cu(act, self.d, block_size, 1) * units
+            deep = groups >= 2 * units and all(step.start_pos[b] >= step.q_lens[b] for b in step.prefill_seqs)
+            if not (fills or deep):
                 per_item = ops.prefill_rows_per_item(act, self.d, block_size, 1)
                 rows = prefill_work_rows(step.q_lens, step.prefill_seqs, G, per_item, step.start_pos)
             found = (step.upload_ints([x for row in rows for x in row]).view(-1, 3), per_item)

@@ -42,17 +42,17 @@ def test_flat_varlen_batch_reference_vector():
         assert slot == cache.slot("ab"[s], p)
     assert step.n_decode == 1 and step.decode_seq_ids.tolist() == [1] and step.prefill_seqs == [0]
     assert step.decode_shape == DecodeShape(n=1, max_ctx=2, sum_ctx=2)
-    # attention's work list for the run of 3 tokens: 3 tokens x group size over 16-row items is
-    # one item, then two paired into one row
+    # attention's work list for the run of 3 tokens: 3 tokens x group size over items of 16 or
+    # 4 rows, one item per row, the longest walk (the last item) first
     from kvforge_amd.parts.attention import prefill_work_rows
     assert prefill_work_rows(step.q_lens, step.prefill_seqs, 2, 16) == [(0, 0, -1)]
-    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 16) == [(0, 0, 1)]
-    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 4) == [(0, 0, 4), (0, 1, 3), (0, 2, -1)]
-    # a run half as far into its sequence as it is long, or farther, is not paired: one item
-    # per workgroup, the last (longest walk) first; a run nearer the start stays in pairs
+    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 16) == [(0, 0, -1), (0, 1, -1)]   # both end in the last token
+    assert prefill_work_rows(step.q_lens, step.prefill_seqs, 6, 4) == [(0, 3, -1), (0, 4, -1), (0, 1, -1), (0, 2, -1), (0, 0, -1)]
+    # several runs: by the keys an item walks, those before its run included; equal walks stay
+    # in sequence order
     q_lens = [3, 3, 1]
     assert prefill_work_rows(q_lens, [0, 1], 6, 4, start_pos=[2, 1, 9]) == \
-        [(0, 4, -1), (0, 3, -1), (0, 2, -1), (0, 1, -1), (0, 0, -1), (1, 0, 4), (1, 1, 3), (1, 2, -1)]
+        [(0, 3, -1), (0, 4, -1), (0, 1, -1), (0, 2, -1), (1, 3, -1), (1, 4, -1), (0, 0, -1), (1, 1, -1), (1, 2, -1), (1, 0, -1)]
 
 
 def test_wanted_places_and_modes():
