@@ -770,6 +770,19 @@ def test_attn_prefill(dtype, seq_lens, q_lens, H, KV, d, bs, window):
         torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
 
 
+def test_prefill_kernel_says_how_many_workgroups_a_compute_unit_holds():
+    """What the planner of query runs weighs rows per item against: asked of the runtime for the
+    kernel that would run, at least one, never more with two row tiles than with one; sizes the
+    matrix-core kernel does not take answer through the 32-bit kernel's constant."""
+    o = ops()
+    for d in (16, 64, 80, 128, 192, 256):
+        one = o.prefill_blocks_per_cu(torch.bfloat16, d, 16, 1)
+        two = o.prefill_blocks_per_cu(torch.bfloat16, d, 16, 2)
+        assert 1 <= two <= one <= 8, (d, one, two)
+    assert o.prefill_blocks_per_cu(torch.float32, 64, 16, 1) >= 1
+    assert o.prefill_blocks_per_cu(torch.bfloat16, 64, 4, 1) >= 1    # pages of 4: the 32-bit kernel's way
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 4), (3, 1, 32, 8), (6, 1, 48, 16),
                                         (4, 4, 80, 16), (32, 8, 64, 16), (8, 2, 128, 16),

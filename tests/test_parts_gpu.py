@@ -169,6 +169,35 @@ def test_attention_part_over_portions(dtype, H, KV, d, window, bs, small_chip, m
         torch.testing.assert_close(torch.cat(got[rid]), want[rid], **tol(dtype))
 
 
+@pytest.mark.parametrize("d,runs,rows_per_item", [
+    (64, [(2048, 0)], 64),            # 512 workgroups of two tiles would leave half the chip's places empty
+    (64, [(4096, 0)], 128),           # 1,024 of them fill it
+    (64, [(2048, 2048)], 128),        # all items walk long: two a compute unit are enough
+    (64, [(2048, 1024)], 64),         # the run starts less than its own length into its sequence
+    (64, [(1024, 0)] * 4, 128),       # several runs count together
+    (128, [(2048, 0)], 64),
+    (128, [(4096, 0)], 128),
+])
+def test_attention_plans_rows_per_item_by_what_fills_the_chip(d, runs, rows_per_item, monkeypatch):
+    """32 heads over 8 kv heads on a chip of 256 compute units: the planner's choice between one
+    and two row tiles per wave, and its order (longest walk first)."""
+    from types import SimpleNamespace
+    from kvforge_amd.kernels import ops as kernel_ops
+    monkeypatch.setattr(kernel_ops, "_compute_units", {i: 256 for i in range(torch.cuda.device_count())})
+    part = PagedAttention("a", 2048, 32, 8, d, RotaryPositions(d, 1000.0))
+    step = SimpleNamespace(q_lens=[n for n, _ in runs], start_pos=[s for _, s in runs],
+                           prefill_seqs=list(range(len(runs))), scratch={}, device=torch.device(DEV),
+                           upload_ints=lambda v: torch.tensor(v, dtype=torch.int32))
+    rows, per_item = part._prefill_work(step, torch.bfloat16, 16)
+    assert per_item == rows_per_item
+    rows = rows.tolist()
+    assert len(rows) == sum(-(-n * 4 // per_item) for n, _ in runs) and all(r[2] == -1 for r in rows)
+    ends = [runs[b][1] + min(runs[b][0], -(-(i + 1) * per_item // 4)) for b, i, _ in rows]
+    assert ends == sorted(ends, reverse=True)
+    assert sorted((b, i) for b, i, _ in rows) == [(b, i) for b, (n, _) in enumerate(runs)
+                                                  for i in range(-(-n * 4 // per_item))]
+
+
 class ToyQKNormAttention(PagedAttention):
     """Attention with a bias on the q projection and an RMS norm per head of q and of k before
     the rotation, added from here through ``after_projection``: the framework's files know of
