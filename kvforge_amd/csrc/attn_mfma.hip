@@ -30,9 +30,13 @@
 // cleared by a mask when it is consumed, so nothing waits on a load before its data is needed.
 //
 // Query runs: an item is 4 * RT consecutive row tiles of one (sequence, kv head), one tile set per
-//   wave; a workgroup takes the items of a work row in turn: the host pairs an early item with a
-//   late one, so that under the causal mask every workgroup walks about as many keys.  Three
-//   stages are in flight: page lookups two blocks ahead, fragment loads one block ahead
+//   wave; a workgroup takes the one or two items of a work row in turn (two: an early item with
+//   a late one, so that under the causal mask every workgroup walks about as many keys; one, the
+//   longest walks first in the grid, keeps more workgroups in flight and is what the engine's
+//   planner hands out).  The kv head is the grid's fastest index where the grid allows it:
+//   consecutive workgroups go to consecutive XCDs, so with eight kv heads an XCD walks the keys
+//   of one head only and finds them in its own L2.  Three or four stages are in
+//   flight: page lookups two or three blocks ahead, fragment loads one or two blocks ahead
 //   (registers, then the other half of a double LDS buffer), products of this block.
 // Few rows, long key range: a workgroup takes one row tile and one of `splits` cuts of the key
 //   range; blocks of 32 keys go round the waves (eight, or four where the grid fills the chip) of
@@ -312,8 +316,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   const int j16 = lane % 16, kg = lane / 16;
   const int G = a.H / a.KV, D = a.d;
   // A work row names a sequence and up to two of its items (the second may be -1), which the
-  // workgroup takes one after the other: the host pairs an early item (few keys to walk) with a
-  // late one (many), so that under the causal mask all workgroups have about the same to do.
+  // workgroup takes one after the other.
   const int wrow = a.kv_fastest ? blockIdx.y : blockIdx.x, kvh = a.kv_fastest ? blockIdx.x : blockIdx.y;
   const int seq = work[3 * wrow];
   if (seq < 0 || seq >= a.n_seqs) return;

@@ -695,7 +695,7 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
     were made; by default its answer for one row tile), and the items of one row are taken by
-    one workgroup in turn (pair an early item with a late one).  ``v_pages`` are transposed:
+    one workgroup in turn; rows start in the order given (the longest walks first).  ``v_pages`` are transposed:
     ``[num_blocks, KV, head_dim, block_size]``.  ``slopes``: fp32 ``[H]``; the score of key ``j``
     for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``."""
     H, KV, d = num_heads, num_kv_heads, head_dim
