@@ -61,6 +61,45 @@ def test_replay_all_modes(tmp_path, name, dtype, store, sharp):
     ru.compare(folder, tb, out, names, atol, rtol)
 
 
+ODD = {  # sizes off every beaten path: head sizes in steps of 16 up to 256, odd numbers of heads and
+    # groups, widths that are multiples of 8 only, prime vocabularies, pages of 8, 24 and 32 tokens
+    "d112": (dict(head_dim=112, num_key_value_heads=5, num_attention_heads=5, hidden_size=104,
+                  intermediate_size=600, vocab_size=4099, num_hidden_layers=2, tie_word_embeddings=False,
+                  layer_types=["sliding_attention", "full_attention"], sliding_window=33), 32),
+    "d144": (dict(head_dim=144, num_key_value_heads=3, num_attention_heads=27, hidden_size=520,
+                  intermediate_size=100, vocab_size=5003, num_hidden_layers=3, tie_word_embeddings=False,
+                  layer_types=["full_attention", "sliding_attention", "full_attention"], sliding_window=24,
+                  rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                                "high_freq_factor": 4.0, "original_max_position_embeddings": 64}), 8),
+    "d256": (dict(head_dim=256, num_key_value_heads=3, num_attention_heads=12, hidden_size=72,
+                  intermediate_size=24, vocab_size=9001, num_hidden_layers=1, tie_word_embeddings=True,
+                  layer_types=["full_attention"]), 16),
+    "d16": (dict(head_dim=16, num_key_value_heads=7, num_attention_heads=49, hidden_size=520,
+                 intermediate_size=600, vocab_size=8999, num_hidden_layers=1, tie_word_embeddings=True,
+                 layer_types=["sliding_attention"], sliding_window=64, rms_norm_eps=3e-4), 24),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", sorted(ODD))
+def test_replay_sizes_that_no_kernel_was_tuned_for(tmp_path, dtype, which):
+    """All four ways of cutting the requests, against the plain model, on shapes that the
+    configuration allows and nothing was built around: each kernel takes them or a slower one
+    does, never a wrong result."""
+    change, block_size = ODD[which]
+    cfg = dict(ru.TINY_C, max_position_embeddings=512, **change)
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, cfg, seed=len(which), dtype=dtype)
+    ru.sharpen(folder, 4.0)
+    prompts = ru.random_prompts(cfg["vocab_size"], [37, 64, 81, 100], 3)
+    tb, names = build_all_modes(prompts, 3)
+    out = str(tmp_path / "out")
+    ru.run_trace(folder, dtype, tb, out, user_args=["--block-size", str(block_size)])
+    atol, rtol = TOL[dtype]
+    ru.compare(folder, tb, out, names, atol, rtol,
+               measured_rounding="bfloat16" if dtype == "bfloat16" else False)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("which", ["WIDE", "WIDE_B", "WIDE_C"])
 def test_replay_layers_wide_enough_for_the_serving_kernels(tmp_path, dtype, which):
