@@ -104,7 +104,8 @@ def _find_built(name: str, want_hash: str) -> str | None:
 
 
 def _log(msg: str) -> None:
-    print(f"[kvforge_amd] {msg}", file=sys.stderr, flush=True)
+    sys.stderr.write(f"[kvforge_amd] {msg}\n")   # one write: lines of modules built side by side stay whole
+    sys.stderr.flush()
 
 
 def build_module(name: str, force: bool = False, verbose: bool = True) -> str:
