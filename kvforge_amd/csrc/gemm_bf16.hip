@@ -39,7 +39,8 @@
 // A product that is added to a narrow C over a long K (the down projection) has fewer workgroups
 // than the chip has compute units, and a compute unit keeps only so many bytes in flight.  It
 // may be cut into two halves of K (`Riders::half_out`): a second layer of workgroups stores its
-// half beside C, and the caller owes that half to C.  The next consumers add it on their way:
+// half beside C (rounded to bf16, as a product that is stored is), and the caller owes that half
+// to C.  The next consumers add it on their way:
 // the fused q/k/v projection in its loads (`a_add`), the output projection in its sum (`c_add`).
 //
 // Layout of W.  In the checkpoint's row-major [N, K] a wave's load of one operand fragment
@@ -66,15 +67,18 @@ struct RopeEpi {
   int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
 };
 
-// Sums that ride along.  `a_add` (kernels built with ADD): the left operand is A + a_add, both
-// fp32 with the same row stride.  `c_add` (with EPI 2): C += product + c_add, same row stride as C.
+// Sums that ride along, all bf16 (a workgroup of the fused projection reads every row of A and
+// of a_add: with the addend in fp32 that was as many bytes again as A, 1.8 us of a 8.6 us kernel
+// at eight rows).  `a_add` (kernels built with ADD): the left operand is A + a_add, A in fp32,
+// the same row stride counted in elements.  `c_add` (with EPI 2): C += product + c_add, row
+// stride of C.
 // `half_out` (with EPI 2): the grid is two deep; workgroups of the second layer walk the second
 // half of K and store their product there (fp32, row stride of C) instead of adding it to C, so
 // that a narrow C still puts a workgroup on every compute unit; the caller owes half_out to C.
 struct Riders {
-  const float* a_add;
-  const float* c_add;
-  float* half_out;
+  const bf16_t* a_add;
+  const bf16_t* c_add;
+  bf16_t* half_out;
 };
 
 // Operands of the greedy pick (EPI 5).  part_val / part_idx: [16][workgroups] and behind them
@@ -222,14 +226,18 @@ __device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
 // Nothing inside the branches uses what they load, so no branch ends in a wait and the loads of
 // a whole pass stay in flight together.
 template <bool ADD>
-__device__ __forceinline__ bf16x8 load_frag_f32(const float* p, const float* q, bool ok, float& ss) {
+__device__ __forceinline__ bf16x8 load_frag_f32(const float* p, const bf16_t* q, bool ok, float& ss) {
   typedef __attribute__((ext_vector_type(8))) float f32x8;
   float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  float w[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  uint4 raw = make_uint4(0u, 0u, 0u, 0u);   // eight bf16 of q, widened after the branch
   if (ok) {
     load8(p, v);
-    if (ADD) load8(q, w);
+    if (ADD) raw = *reinterpret_cast<const uint4*>(q);
   }
+  const float w[8] = {__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
+                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u),
+                      __uint_as_float(raw.z << 16), __uint_as_float(raw.z & 0xffff0000u),
+                      __uint_as_float(raw.w << 16), __uint_as_float(raw.w & 0xffff0000u)};
   f32x8 x;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -260,17 +268,22 @@ __device__ __forceinline__ bool vec4_ok(const void* Cv, int ldc, int n, int N, i
 // First stage: loads that need only (m, n).
 template <int EPI>
 __device__ __forceinline__ void epi_prefetch_a(EpiOperands& op, int m, int n, int N, int ldc, const void* Cv,
-                                               const float* c_add, const RopeEpi& rp) {
+                                               const bf16_t* c_add, const RopeEpi& rp) {
   op.have = true;
   if (EPI == 2) {
     const size_t idx = static_cast<size_t>(m) * ldc + n;
     const float* c = static_cast<const float*>(Cv) + idx;
-    if (vec4_ok(Cv, ldc, n, N, 4) && vec4_ok(c_add, ldc, n, N, 4)) {
+    if (vec4_ok(Cv, ldc, n, N, 4) && vec4_ok(c_add, ldc, n, N, 2)) {
       op.c = *reinterpret_cast<const f32x4*>(c);
-      if (c_add) op.c += *reinterpret_cast<const f32x4*>(c_add + idx);
+      if (c_add) {
+        const uint2 packed = *reinterpret_cast<const uint2*>(c_add + idx);
+        op.c += f32x4{__uint_as_float(packed.x << 16), __uint_as_float(packed.x & 0xffff0000u),
+                      __uint_as_float(packed.y << 16), __uint_as_float(packed.y & 0xffff0000u)};
+      }
     } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) op.c[r] = n + r < N ? c[r] + (c_add ? c_add[idx + r] : 0.f) : 0.f;
+      for (int r = 0; r < 4; ++r)
+        op.c[r] = n + r < N ? c[r] + (c_add ? bf16_to_f32(c_add[idx + r].bits) : 0.f) : 0.f;
     }
   }
   if (EPI == 4) {
@@ -305,7 +318,7 @@ __device__ __forceinline__ void epi_prefetch_b(EpiOperands& op, int n, const Rop
 // One lane's four neighbouring columns n..n+3 of row m, after the waves' partial sums are added.
 template <int EPI>
 __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, int ldc, void* Cv,
-                                           const float* c_add, const RopeEpi& rp, EpiOperands& op) {
+                                           const bf16_t* c_add, const RopeEpi& rp, EpiOperands& op) {
   if (EPI == 2 || EPI == 4) {
     if (!op.have) {
       epi_prefetch_a<EPI>(op, m, n, N, ldc, Cv, c_add, rp);
@@ -425,8 +438,8 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
   }
   const bf16_t* Ab = static_cast<const bf16_t*>(Av);
   const float* Af = static_cast<const float*>(Av);
-  const float* a_add = ADD ? rd.a_add : nullptr;
-  const float* c_add = EPI == 2 && !second ? rd.c_add : nullptr;
+  const bf16_t* a_add = ADD ? rd.a_add : nullptr;
+  const bf16_t* c_add = EPI == 2 && !second ? rd.c_add : nullptr;
   f32x4 acc[NT][MT];
   float ss[MT];
 #pragma unroll
@@ -545,7 +558,7 @@ __global__ __launch_bounds__(max_waves(MT, NT, AT) * KVF_WAVE) void gemm_skinny_
       EpiOperands fresh;
       fresh.have = false;
       if (EPI == 2 && second)
-        store_tile<0>(s, m, n, N, ldc, rd.half_out, nullptr, rp, fresh);
+        store_tile<1>(s, m, n, N, ldc, rd.half_out, nullptr, rp, fresh);
       else
         store_tile<EPI>(s, m, n, N, ldc, Cv, c_add, rp, PRE ? pre[j] : fresh);
     }
@@ -713,19 +726,19 @@ KVF_EXPORT void kvf_gemm_bf16_set_rows(int rows) { g_rows_override = rows; }
 // a_type: 0 = bf16 rows, 1 = fp32 rows normalised by rsqrt(mean(x^2) + eps) in the kernel.
 // epi: 0 store fp32, 1 store bf16, 2 add into fp32, 3 SwiGLU pairs -> bf16 [M, N/2].
 // w_tiled: W is [N, K] row-major (0) or in tiles of 16 x 32 (1, see the head of this file).
-// c_add (epi 2 only, may be null): fp32 [M, ldc], added to C together with the product.
-// half_out (epi 2 with bf16 rows only, may be null): fp32 [M, ldc]; the product over the second
+// c_add (epi 2 only, may be null): bf16 [M, ldc], added to C together with the product.
+// half_out (epi 2 with bf16 rows only, may be null): bf16 [M, ldc]; the product over the second
 //   half of K is stored there instead of being added to C, by a second layer of workgroups.
 KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, int w_tiled, void* C, int epi,
-                             int M, int N, int K, int lda, int ldc, float eps, const float* c_add,
-                             float* half_out, hipStream_t s) {
+                             int M, int N, int K, int lda, int ldc, float eps, const void* c_add,
+                             void* half_out, hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || epi < 0 || epi > 3 || (epi == 3 && N % 4 != 0))
     return static_cast<int>(hipErrorInvalidValue);
   if (((c_add || half_out) && epi != 2) || (half_out && (a_type != 0 || K < 64)))
     return static_cast<int>(hipErrorInvalidValue);
   const RopeEpi none{};
-  const Riders rd{nullptr, c_add, half_out};
+  const Riders rd{nullptr, static_cast<const bf16_t*>(c_add), static_cast<bf16_t*>(half_out)};
   const bf16_t* w = static_cast<const bf16_t*>(W);
   if (a_type == 0) return launch_epi<0>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, rd, none, s);
   if (a_type == 1) return launch_epi<1>(A, w, C, epi, M, N, K, lda, ldc, eps, w_tiled, rd, none, s);
@@ -734,11 +747,11 @@ KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, int w_til
 
 // Fused q/k/v projection with rotary and cache write.  W: [(H + 2*KV) * d, K] with q and k rows
 // permuted so that rotary pairs are neighbouring rows.  q_out: [M, ldq >= H * d] bf16.
-// a_add (a_type 1 and at most 16 rows only, may be null): fp32 [M, lda], added to A before the
+// a_add (a_type 1 and at most 16 rows only, may be null): bf16 [M, lda], added to A before the
 // norm.
 KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, int w_tiled,
                                       void* q_out, int M, int K, int lda, int ldq, float eps,
-                                      const float* a_add, const int* positions,
+                                      const void* a_add, const int* positions,
                                       const int* seq_of_token, const float* cos_t,
                                       const float* sin_t, const int* block_table, void* k_pages,
                                       void* v_pages, int H, int KV, int d, int rot, int table_len,
@@ -748,7 +761,7 @@ KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, 
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || d % 4 != 0 || rot % 2 != 0 || rot > d || ldq % 4 != 0 ||
       (a_add && (a_type != 1 || M > 16)))
     return static_cast<int>(hipErrorInvalidValue);
-  const Riders rd{a_add, nullptr, nullptr};
+  const Riders rd{static_cast<const bf16_t*>(a_add), nullptr, nullptr};
   const RopeEpi rp{positions, seq_of_token, cos_t, sin_t, block_table,
                    static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), H, KV, d, rot,
                    table_len, block_size, table_stride, num_blocks, write_kv, n_seqs};

@@ -411,10 +411,10 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
     ``out: [M, N]``.
     bf16 x bf16 runs on MFMA with fp32 accumulation; any operand in fp32 runs the fp32
     vector-ALU kernel (true 32-bit multiply and accumulate).
-    With ``accumulate``: ``owed`` (fp32, like ``out``) is a sum still owed to ``out`` and is added
-    on the way; ``half_out`` (fp32, like ``out``, only where ``k_halves_pay``) receives the
-    product over the second half of K *instead of* ``out``, which the caller then owes to
-    ``out``: twice the workgroups pull on ``w``."""
+    With ``accumulate``: ``owed`` (bf16, shape and row stride of ``out``) is a sum still owed to
+    ``out`` and is added on the way; ``half_out`` (bf16, likewise, only where ``k_halves_pay``)
+    receives the product over the second half of K *instead of* ``out``, which the caller then
+    owes to ``out``: twice the workgroups pull on ``w``."""
     m, n, k, lda, ldc = _gemm_operands(a, w, out, lambda n: n)
     if accumulate and out.dtype != F32:
         raise KernelError("gemm: accumulation needs an fp32 output")
@@ -423,7 +423,7 @@ def gemm(a: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False,
             continue
         if not accumulate:
             raise KernelError(f"gemm: {name} goes with accumulate")
-        _check(t, name, F32, (m, n), contiguous=False)
+        _check(t, name, BF16, (m, n), contiguous=False)
         if t.stride(1) != 1 or (m > 1 and t.stride(0) != ldc):
             raise KernelError(f"gemm: {name} must have the row stride of out")
     if half_out is not None and not k_halves_pay(a, w):
@@ -505,8 +505,8 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
                   rms_eps: float | None = None, a_owed: torch.Tensor | None = None) -> None:
     """Fused q/k/v projection: ``a @ w.T`` with rotary applied to q and k (neighbouring columns
     are pairs), rotated q stored to ``q_out [M, H*d]`` and rotated k and v written into the
-    pages; without tables (``None``) nothing is rotated.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; fp32, shape and
-    strides of ``a``): a sum still owed to ``a``; the projection is taken of ``a + a_owed``, and
+    pages; without tables (``None``) nothing is rotated.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; bf16, shape and
+    strides, counted in elements, of ``a``): a sum still owed to ``a``; the projection is taken of ``a + a_owed``, and
     ``a`` itself is left as it is."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     rms = rms_eps is not None
@@ -518,7 +518,7 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     if a_owed is not None:
         if not rms or m > FUSED_NORM_MAX_M:
             raise KernelError("gemm_qkv_rope: a_owed goes with rms_eps (fp32 rows, one tile of them)")
-        _check(a_owed, "a_owed", F32, (m, k), contiguous=False)
+        _check(a_owed, "a_owed", BF16, (m, k), contiguous=False)
         if a_owed.stride() != a.stride():
             raise KernelError("gemm_qkv_rope: a_owed must have the strides of a")
     _check(q_out, "q_out", BF16, (m, H * d))

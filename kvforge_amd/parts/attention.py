@@ -249,10 +249,10 @@ class PagedAttention(Mixer):
         fused = (not self._hooked() and ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
                  and layer.k_pages.dtype == torch.bfloat16)
         if fused and rms is not None:
-            # what the layer before owes the stream in fp32 rides in this projection's loads and
-            # is added to the stream by the output projection
+            # what the layer before owes the stream rides in this projection's loads and is
+            # added to the stream by the output projection
             owed = step.take_owed(residual)
-            if owed is not None and owed.dtype != torch.float32:
+            if owed is not None and (owed.dtype != torch.bfloat16 or owed.stride() != x.stride()):
                 ops.add_rows(residual, owed)
                 owed = None
         else:

@@ -286,7 +286,7 @@ def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.
     product is left owed to the stream (``step.owe``) so that the next norm adds it on its way
     instead of an add kernel of its own.  One tile of rows over a deep weight with few columns
     is cut into two halves of K so that every compute unit pulls on the weight: the first half
-    is added here, the second is left owed (in fp32).
+    is added here, the second is left owed (rounded to bf16, as a stored product is).
     ``owed``: a sum the caller took from the step (``step.take_owed``) and has not added yet;
     it is added here, in the same kernel where that is possible."""
     from kvforge_amd.kernels import ops
@@ -298,12 +298,12 @@ def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.
         ops.gemm(a, w, product)
         step.owe(residual, product)
     elif ops.k_halves_pay(a, w) and residual.is_contiguous():
-        half = step.ws.buf("owed_half", tuple(residual.shape), torch.float32)
+        half = step.ws.buf("owed_half", tuple(residual.shape), torch.bfloat16)
         if owed is not None and owed.data_ptr() == half.data_ptr():
             # what the caller took from the step is the half the product before this one left
             # there: this product's workgroups read it while others write their half, so the
             # new half goes to the other of two buffers
-            half = step.ws.buf("owed_half_other", tuple(residual.shape), torch.float32)
+            half = step.ws.buf("owed_half_other", tuple(residual.shape), torch.bfloat16)
         ops.gemm(a, w, residual, accumulate=True, owed=owed, half_out=half)
         step.owe(residual, half)
     else:

@@ -45,7 +45,7 @@ def test_embed(dtype):
 @pytest.mark.parametrize("add32", [False, True])
 def test_rmsnorm_with_owed_sum(dtype, h, add32):
     """norm(x + add): without rows the sum is left in x; with rows x stays as it was.  The sum
-    owed is in the output's type (a library product) or in fp32 (half of a product cut in K)."""
+    owed is in the output's type (a library product, half of a product cut in K) or in fp32."""
     g = torch.Generator().manual_seed(h + 1)
     x = torch.randn(7, h, generator=g) * 2
     add = torch.randn(7, h, generator=g).to(torch.float32 if add32 else dtype)
@@ -220,7 +220,7 @@ def test_gemm_of_many_rows_through_the_library_entry_point(m, n, k):
     ops().gemm(av, w, outb)
     torch.testing.assert_close(outb.double().cpu(), want, atol=2e-2, rtol=2e-2)
     # a sum still owed to the stream is added by the engine's own kernel on the way
-    owed = torch.randn(m, n, generator=g)
+    owed = torch.randn(m, n, generator=g).to(torch.bfloat16)
     acc = res.clone().to(DEV)
     ops().gemm(av, w, acc, accumulate=True, owed=owed.to(DEV))
     torch.testing.assert_close(acc.double().cpu(), res.double() + owed.double() + want, atol=1e-4, rtol=1e-4)
@@ -332,25 +332,26 @@ def test_gemm_over_tiled_weights_gives_the_same_bits(m, n, k):
 @pytest.mark.parametrize("n,k", [(2048, 8192), (100, 4096), (1040, 4104)])
 @pytest.mark.parametrize("tiled", [False, True])
 def test_gemm_cut_in_two_halves_of_k(m, n, k, tiled):
-    """out += a @ w.T with the second half of K left in half_out, and a sum owed to out added on
-    the way: out + half_out is the whole sum; every value is an fp32 sum in a fixed order, so a
-    second call gives the same bits."""
+    """out += a @ w.T with the second half of K left in half_out (bf16: rounded once, as a stored
+    product is), and a sum owed to out (bf16 too) added on the way: out + half_out is the whole
+    sum; every value is an fp32 sum in a fixed order, so a second call gives the same bits."""
     g = torch.Generator().manual_seed(m + n + k)
     a = torch.randn(m, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / k ** 0.5).to(torch.bfloat16).to(DEV)
     w = ops().StreamedWeight(w) if tiled else w
     res = torch.randn(m, n, generator=g)
-    owed = torch.randn(m, n, generator=g)
+    owed = torch.randn(m, n, generator=g).to(torch.bfloat16)
     assert ops().k_halves_pay(a.to(DEV), w)
     cut = (-(-k // 32) + 1) // 2 * 32                    # the first half takes the odd k-step
     first = a[:, :cut].double() @ ops().plain_of(w).cpu()[:, :cut].double().T
     second = a[:, cut:].double() @ ops().plain_of(w).cpu()[:, cut:].double().T
     outs = []
     for _ in range(2):
-        out, half = res.clone().to(DEV), torch.full((m, n), 7.0, device=DEV)
+        out, half = res.clone().to(DEV), torch.full((m, n), 7.0, device=DEV, dtype=torch.bfloat16)
         ops().gemm(a.to(DEV), w, out, accumulate=True, owed=owed.to(DEV), half_out=half)
         torch.testing.assert_close(out.double().cpu(), res.double() + owed.double() + first, atol=1e-4, rtol=1e-4)
-        torch.testing.assert_close(half.double().cpu(), second, atol=1e-4, rtol=1e-4)
+        # the half is the 32-bit sum rounded to bfloat16 once: within half a unit of its last place
+        torch.testing.assert_close(half.double().cpu(), second, atol=1e-4, rtol=2.0 ** -8)
         outs.append((out, half))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     # the sum owed alone, without the cut
@@ -359,10 +360,12 @@ def test_gemm_cut_in_two_halves_of_k(m, n, k, tiled):
     torch.testing.assert_close(out.double().cpu(), res.double() + owed.double() + first + second,
                                atol=1e-4, rtol=1e-4)
     with pytest.raises(ops().KernelError):
-        ops().gemm(a.to(DEV), w, torch.empty(m, n, device=DEV), half_out=torch.empty(m, n, device=DEV))
+        ops().gemm(a.to(DEV), w, torch.empty(m, n, device=DEV), half_out=torch.empty(m, n, device=DEV, dtype=torch.bfloat16))
     with pytest.raises(ops().KernelError):               # a shallow weight is not cut
         ops().gemm(a.to(DEV)[:, :64].contiguous(), ops().plain_of(w)[:, :64].contiguous(), res.clone().to(DEV),
-                   accumulate=True, half_out=torch.empty(m, n, device=DEV))
+                   accumulate=True, half_out=torch.empty(m, n, device=DEV, dtype=torch.bfloat16))
+    with pytest.raises(ops().KernelError):               # sums that ride along are bfloat16
+        ops().gemm(a.to(DEV), w, res.clone().to(DEV), accumulate=True, owed=owed.float().to(DEV))
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 20, 33, 50, 64])
@@ -470,14 +473,14 @@ def test_gemm_qkv_rope_equals_the_three_steps(m, H, KV, d, rot, bs, rms):
     if rms:
         # a sum still owed to the rows rides in the loads: the same bits as rows summed before,
         # and the rows themselves stay as they were
-        a1, a2 = torch.randn(m, k, generator=g), torch.randn(m, k, generator=g)
+        a1, a2 = torch.randn(m, k, generator=g), torch.randn(m, k, generator=g).to(torch.bfloat16)
         got = []
-        for rows, owed in (((a1 + a2).to(DEV), None), (a1.to(DEV), a2.to(DEV))):
+        for rows, owed in (((a1 + a2.float()).to(DEV), None), (a1.to(DEV), a2.to(DEV))):
             kp2, vp2, q2 = torch.zeros_like(kp_ref), torch.zeros_like(vp_ref), torch.empty_like(q)
             ops().gemm_qkv_rope(rows, w, q2, positions.to(DEV), seq_of.to(DEV), cos_t, sin_t, table.to(DEV),
                                 kp2, vp2, H, KV, d, rms_eps=eps, a_owed=owed)
             got.append((q2, kp2.cpu()[sel], vp2.cpu()[sel_v]))
-            assert torch.equal(rows.cpu(), a1 if owed is not None else a1 + a2)
+            assert torch.equal(rows.cpu(), a1 if owed is not None else a1 + a2.float())
         assert all(torch.equal(x1, x2) for x1, x2 in zip(*got))
 
 
