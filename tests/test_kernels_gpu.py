@@ -602,8 +602,8 @@ def test_gemm_generic_few_rows_over_long_and_uneven_k(m, tw):
     torch.testing.assert_close(acc.double(), want + 1.0, atol=3e-5, rtol=1e-5)
 
 
-@pytest.mark.parametrize("ta", DTYPES)
-@pytest.mark.parametrize("tw", DTYPES)
+# bf16 x bf16 with many rows is the library's or the bf16 kernel's product: not among the pairs
+@pytest.mark.parametrize("ta,tw", [(a, w) for a in DTYPES for w in DTYPES if torch.float32 in (a, w)])
 @pytest.mark.parametrize("mnk", [(33, 130, 96), (200, 70, 260), (129, 257, 2052), (300, 1000, 64),
                                  (128, 128, 32), (260, 4100, 36)])
 def test_gemm_generic_many_rows_on_the_matrix_cores(ta, tw, mnk):
@@ -613,8 +613,6 @@ def test_gemm_generic_many_rows_on_the_matrix_cores(ta, tw, mnk):
     storing and adding into the stream.  A row's result does not depend on the rows around it, and
     the kernel of the vector ALUs, kept for this comparison, agrees to rounding."""
     m, n, k = mnk
-    if ta == tw == torch.bfloat16:
-        pytest.skip("bf16 x bf16 with many rows is the library's or the bf16 kernel's product")
     g = torch.Generator().manual_seed(m + n + k)
     a = torch.randn(m, k, generator=g).to(ta).to(DEV)
     w = (torch.randn(n, k, generator=g) * 0.1).to(tw).to(DEV)
