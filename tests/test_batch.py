@@ -201,3 +201,23 @@ def test_what_a_part_sends_along_with_a_step():
     got = step.upload_ints([(0, 1, -1), (0, 0, 2)])
     assert got.dtype == torch.int32 and got.tolist() == [0, 1, -1, 0, 0, 2]
     assert meta.total == meta.extra_off + meta.extra_size and meta.extra_size >= 4 * 64
+
+
+def test_prefill_work_rows_hold_every_item_once_longest_walk_first():
+    """Random runs, group sizes and item sizes: every item of every run longer than one token
+    appears once, alone in its row, and the rows never go from a shorter walk to a longer one."""
+    import random
+    from kvforge_amd.parts.attention import prefill_work_rows
+    rng = random.Random(5)
+    for _ in range(200):
+        n = rng.randint(1, 6)
+        q_lens = [rng.choice([1, 1, 2, 3, 17, 64, 200, 1000]) for _ in range(n)]
+        start = [rng.choice([0, 0, 5, 64, 999]) for _ in range(n)]
+        seqs = [b for b in range(n) if q_lens[b] > 1]
+        group, per_item = rng.choice([1, 2, 3, 4, 7, 8]), rng.choice([64, 128])
+        rows = prefill_work_rows(q_lens, seqs, group, per_item, start)
+        assert all(second == -1 for _, _, second in rows)
+        want = sorted((b, i) for b in seqs for i in range(-(-q_lens[b] * group // per_item)))
+        assert sorted((b, i) for b, i, _ in rows) == want
+        ends = [start[b] + min(q_lens[b], -(-(i + 1) * per_item // group)) for b, i, _ in rows]
+        assert ends == sorted(ends, reverse=True)
